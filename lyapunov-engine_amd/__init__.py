@@ -1,4 +1,4 @@
-"""An inference engine for decoder-only language models (Llama, Faledra, Ronupel) on one AMD MI355X (gfx950).
+"""An inference engine for decoder-only language models (Llama, Faledra, Ronupel, Tonilix) on one AMD MI355X (gfx950).
 
 From a model folder (config.json, safetensors) to generated tokens: typed
 configuration and registry (``config``), weights by tensor name (``weights``),

@@ -340,6 +340,79 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
   }
 }
 
+// ------------------------------------------------------- choice within groups
+// Sigmoid scores s = sigmoid(x W^T) in 32-bit; the choice goes by s + correction, the weights by s
+// alone.  The experts form n_groups equal groups of neighbours; a group's score is the sum of its
+// two largest choice scores (its one score when a group is one expert), and only experts of the
+// `keep` best groups can be chosen.  The `top` largest choice scores among those are taken (of
+// equal ones the first); their weights are s over the sum of the chosen s (+ 1e-20), times scale.
+// One wave per row: the lanes share the inner dimension of every expert's product in a fixed
+// order, lane 0 then chooses.
+constexpr int kGroupedRows = 4;   // rows (waves) a workgroup
+
+template <typename T>
+__global__ __launch_bounds__(kGroupedRows* kWave) void moe_route_grouped_kernel(
+    const T* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ correction, int rows, int E,
+    int K, int top, int n_groups, int keep, float scale, int32_t* __restrict__ idx, float* __restrict__ wgt) {
+  __shared__ float s_score[kGroupedRows][kMostExperts];    // s
+  __shared__ float s_choice[kGroupedRows][kMostExperts];   // s + correction
+  __shared__ int s_open[kGroupedRows][kMostExperts];       // 1: may still be chosen
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int row = blockIdx.x * kGroupedRows + wave;
+  if (row >= rows) return;
+  const T* xr = x + static_cast<size_t>(row) * ldx;
+  for (int e = 0; e < E; ++e) {
+    const float* we = w + static_cast<size_t>(e) * K;
+    float acc = 0.f;
+    for (int k = lane; k < K; k += kWave) acc += to_f32(xr[k]) * we[k];
+    acc = wave_sum(acc);
+    if (lane == 0) {
+      const float s = 1.0f / (1.0f + expf(-acc));
+      s_score[wave][e] = s;
+      s_choice[wave][e] = s + (correction != nullptr ? correction[e] : 0.f);
+      s_open[wave][e] = 0;
+    }
+  }
+  if (lane != 0) return;
+  const float* c = s_choice[wave];
+  int* open = s_open[wave];
+  const int per = E / n_groups;
+  float gscore[64];   // there are at most 64 groups
+  for (int g = 0; g < n_groups; ++g) {
+    float a = LYP_NEG_INF, b = LYP_NEG_INF;   // the two largest
+    for (int i = 0; i < per; ++i) {
+      const float v = c[g * per + i];
+      if (v > a) {
+        b = a;
+        a = v;
+      } else if (v > b) {
+        b = v;
+      }
+    }
+    gscore[g] = per > 1 ? a + b : a;
+  }
+  unsigned long long taken = 0ull;
+  for (int n = 0; n < keep; ++n) {
+    int best = -1;
+    for (int g = 0; g < n_groups; ++g)
+      if (!((taken >> g) & 1ull) && (best < 0 || gscore[g] > gscore[best])) best = g;
+    taken |= 1ull << best;
+    for (int i = 0; i < per; ++i) open[best * per + i] = 1;
+  }
+  float total = 0.f;
+  for (int n = 0; n < top; ++n) {
+    int best = -1;
+    for (int e = 0; e < E; ++e)
+      if (open[e] && (best < 0 || c[e] > c[best])) best = e;
+    open[best] = 0;
+    idx[static_cast<size_t>(row) * top + n] = best;
+    total += s_score[wave][best];
+  }
+  for (int n = 0; n < top; ++n)
+    wgt[static_cast<size_t>(row) * top + n] = s_score[wave][idx[static_cast<size_t>(row) * top + n]] / (total + 1e-20f) * scale;
+}
+
+
 // ------------------------------------------------------------------- product
 // Two kernels: tiles of up to 16 rows for experts that see few rows (moe_gemm_few_kernel), tiles of
 // 128 rows through LDS on the 32x32 instruction for experts that see many (moe_gemm_wide_kernel).
@@ -352,6 +425,9 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
 // operands straight from memory into the matrix instruction's registers, four steps' loads in flight,
 // and add their sums up through LDS in the order of the waves.
 constexpr int kFewAhead = 4;
+// what a product without a gate may do besides: take its rows by token (as a gated one does) and square
+// the positive part of its result
+enum MoeFlags : int { kMoeGather = 1, kMoeRelu2 = 2 };
 
 template <typename T, bool GATED>
 __global__ __launch_bounds__(256) void moe_gemm_few_kernel(
@@ -359,7 +435,7 @@ __global__ __launch_bounds__(256) void moe_gemm_few_kernel(
     T* __restrict__ out, int ldo, const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
     const int32_t* __restrict__ n_tiles, const int32_t* __restrict__ expert_off,
     const int32_t* __restrict__ sorted_pair, int top, int N, int K, int up_offset, float limit, float alpha,
-    int vec_ok) {
+    int vec_ok, int flags) {
   using MW = Mma16Wide<T>;
   constexpr int KE = MW::kElems, STEP = 4 * KE;
   __shared__ float s_red[4][2][kWave][4];
@@ -375,7 +451,7 @@ __global__ __launch_bounds__(256) void moe_gemm_few_kernel(
   const T* we = w + static_cast<size_t>(e) * w_expert_stride;
   const int place = row0 + r;
   const T* x_row = nullptr;
-  if (place < row_end) x_row = a + static_cast<size_t>(GATED ? sorted_pair[place] / top : place) * lda;
+  if (place < row_end) x_row = a + static_cast<size_t>((GATED || (flags & kMoeGather)) ? sorted_pair[place] / top : place) * lda;
   const int col = c0 + r;
   const T* g_row = col < N ? we + static_cast<size_t>(col) * ldw : nullptr;
   const T* u_row = GATED && col < N ? we + static_cast<size_t>(col + up_offset) * ldw : nullptr;
@@ -427,6 +503,9 @@ __global__ __launch_bounds__(256) void moe_gemm_few_kernel(
       const float g = fminf(y, limit);
       const float u = fminf(fmaxf(up, -limit), limit);
       y = g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+    } else if (flags & kMoeRelu2) {
+      y = fmaxf(y, 0.f);
+      y *= y;
     }
     orow[c] = from_f32<T>(y);
   }
@@ -451,7 +530,7 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_wide_kernel(
     T* __restrict__ out, int ldo, const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
     const int32_t* __restrict__ n_tiles, const int32_t* __restrict__ expert_off,
     const int32_t* __restrict__ sorted_pair, int top, int N, int K, int up_offset, float limit, float alpha,
-    int vec_ok) {
+    int vec_ok, int flags) {
   using MW = Mma32<T>;
   constexpr int VEC = 16 / sizeof(T);
   constexpr int KT = MoeWide<T, NW>::kKT;             // inner values a round: 128 bytes of every row
@@ -504,7 +583,7 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_wide_kernel(
     a_src[n] = nullptr;
     if (row0 + r < row_end) {
       const int place = row0 + r;
-      a_src[n] = a + static_cast<size_t>(GATED ? sorted_pair[place] / top : place) * lda;
+      a_src[n] = a + static_cast<size_t>((GATED || (flags & kMoeGather)) ? sorted_pair[place] / top : place) * lda;
     }
   }
 #pragma unroll
@@ -616,7 +695,13 @@ __global__ __launch_bounds__(NW * 64) void moe_gemm_wide_kernel(
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           const int col = c0 + wn * 64 + j * 32 + f;
-          if (col < N) orow[col] = from_f32<T>(acc[i][j][v]);
+          if (col >= N) continue;
+          float y = acc[i][j][v];
+          if (flags & kMoeRelu2) {
+            y = fmaxf(y, 0.f);
+            y *= y;
+          }
+          orow[col] = from_f32<T>(y);
         }
       }
     }
@@ -720,6 +805,30 @@ int lyp_moe_route(const float* z, const float* bias, int rows, int E, int top, i
 // x [rows, K] in the activations' type, w [E, K] float: the router's logits, the choice and the weights.
 // How many workgroups had better share a row block's inner dimension (1: none; more need `part`,
 // that many * rows * E floats).
+// x [rows, K] of dtype (rows ldx apart); w float [E, K]; correction float [E] or null; idx int32 and
+// wgt float [rows, top].  n_groups divides E, keep * (E / n_groups) >= top, at most 64 groups.
+int lyp_moe_route_grouped(const void* x, int ldx, int dtype, const float* w, const float* correction, int rows, int E,
+                          int K, int top, int n_groups, int keep, float scale, int32_t* idx, float* wgt,
+                          hipStream_t stream) {
+  LYP_REQUIRE(rows >= 0 && E > 0 && E <= kMostExperts && K > 0 && ldx >= K && top > 0,
+              "moe_route_grouped: %d rows, %d experts (at most %d), inner size %d, %d chosen", rows, E, kMostExperts, K, top);
+  LYP_REQUIRE(n_groups >= 1 && n_groups <= 64 && E % n_groups == 0 && keep >= 1 && keep <= n_groups &&
+                  keep * (E / n_groups) >= top,
+              "moe_route_grouped: %d experts in %d groups of which %d are kept cannot give %d choices", E, n_groups, keep, top);
+  if (rows == 0) return 0;
+  const int blocks = (rows + kGroupedRows - 1) / kGroupedRows;
+  if (dtype == kF32)
+    moe_route_grouped_kernel<float><<<blocks, kGroupedRows * kWave, 0, stream>>>(
+        static_cast<const float*>(x), ldx, w, correction, rows, E, K, top, n_groups, keep, scale, idx, wgt);
+  else if (dtype == kBF16)
+    moe_route_grouped_kernel<bf16_t><<<blocks, kGroupedRows * kWave, 0, stream>>>(
+        static_cast<const bf16_t*>(x), ldx, w, correction, rows, E, K, top, n_groups, keep, scale, idx, wgt);
+  else
+    LYP_REQUIRE(false, "moe_route_grouped: unknown dtype %d", dtype);
+  LYP_LAUNCH_CHECK("moe_route_grouped");
+  return 0;
+}
+
 int lyp_moe_route_splits(int rows, int K) {
   const int blocks = (rows + 15) / 16, steps = (K + 15) / 16;
   int ks = compute_units() / std::max(blocks, 1);
@@ -798,11 +907,12 @@ int lyp_moe_route_sort(const float* part, int parts, const float* bias, int rows
 }
 
 // gated != 0: a [tokens, K] gathered by token, w [E][2 N rows: gates, then ups][K], out [pairs, N] in the
-// operands' type.  gated == 0: a [pairs, K] by place, w [E][N][K], out [pairs, N] in the operands' type.
+// operands' type.  gated == 0: a [pairs, K] by place, w [E][N][K], out [pairs, N] in the operands' type;
+// flags & 1: a [tokens, K] gathered by token instead; flags & 2: the result's positive part squared.
 int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_stride, int ldw, void* out, int ldo,
                  int dtype, int gated, const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* n_tiles,
                  int most_tiles, int tile_rows, const int32_t* expert_off, const int32_t* sorted_pair, int top, int N,
-                 int K, float limit, float alpha, hipStream_t stream) {
+                 int K, float limit, float alpha, int flags, hipStream_t stream) {
   LYP_REQUIRE(N > 0 && K > 0 && lda >= K && ldw >= K && ldo >= N && top > 0 && most_tiles >= 0,
               "moe_gemm: bad sizes N=%d K=%d lda=%d ldw=%d ldo=%d", N, K, lda, ldw, ldo);
   LYP_REQUIRE(tile_rows == 16 || tile_rows == 128, "moe_gemm: tiles of %d rows", tile_rows);
@@ -833,11 +943,11 @@ int lyp_moe_gemm(const void* a, int lda, const void* w, long long w_expert_strid
   }                                                                                                             \
   moe_gemm_wide_kernel<T, G, NWV><<<grid, NWV * 64, MoeWide<T, NWV>::kBytes, stream>>>(                         \
       static_cast<const T*>(a), lda, static_cast<const T*>(w), w_expert_stride, ldw, static_cast<T*>(out), ldo, \
-      tile_expert, tile_row0, n_tiles, expert_off, sorted_pair, top, N, K, N, limit, alpha, vec_ok)
+      tile_expert, tile_row0, n_tiles, expert_off, sorted_pair, top, N, K, N, limit, alpha, vec_ok, flags)
 #define LYP_MOE_FEW(T, G)                                                                                       \
   moe_gemm_few_kernel<T, G><<<grid, 256, 0, stream>>>(                                                          \
       static_cast<const T*>(a), lda, static_cast<const T*>(w), w_expert_stride, ldw, static_cast<T*>(out), ldo, \
-      tile_expert, tile_row0, n_tiles, expert_off, sorted_pair, top, N, K, N, limit, alpha, vec_ok)
+      tile_expert, tile_row0, n_tiles, expert_off, sorted_pair, top, N, K, N, limit, alpha, vec_ok, flags)
 #define LYP_MOE_T(T)                                 \
   do {                                               \
     if (few) {                                       \

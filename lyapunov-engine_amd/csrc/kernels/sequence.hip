@@ -191,11 +191,15 @@ __global__ void branch_join_vec_kernel(float* __restrict__ h, const TY* __restri
 // Work items: one per row (rows whose history lies inside the step), then one
 // per request, which does the rows that read the slot and then rewrites the
 // slot, so that no other thread reads a slot while it changes.
+// The input's rows may lie ldx values apart (a column range of a wider tensor);
+// act != 0: silu of the result (with residual == 0 a plain convolution and its activation).
+__device__ __forceinline__ float conv_silu(float v) { return v / (1.0f + expf(-v)); }
+
 template <typename T>
 __global__ void short_conv_kernel(const T* __restrict__ x, const float* __restrict__ w, T* __restrict__ state,
                                   const int32_t* __restrict__ q_start, const int32_t* __restrict__ positions,
                                   const int32_t* __restrict__ slots, T* __restrict__ out, int n_rows, int B, int C,
-                                  int taps, int residual) {
+                                  int taps, int residual, int ldx, int act) {
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   const int item = blockIdx.x;
   const int hist = taps - 1;
@@ -209,9 +213,9 @@ __global__ void short_conv_kernel(const T* __restrict__ x, const float* __restri
     }
     if (i < hist) return;
     const float* wc = w + static_cast<size_t>(c) * taps;
-    float acc = residual ? to_f32(x[static_cast<size_t>(item) * C + c]) : 0.f;
-    for (int j = 0; j < taps; ++j) acc += wc[j] * to_f32(x[static_cast<size_t>(item - hist + j) * C + c]);
-    out[static_cast<size_t>(item) * C + c] = from_f32<T>(acc);
+    float acc = residual ? to_f32(x[static_cast<size_t>(item) * ldx + c]) : 0.f;
+    for (int j = 0; j < taps; ++j) acc += wc[j] * to_f32(x[static_cast<size_t>(item - hist + j) * ldx + c]);
+    out[static_cast<size_t>(item) * C + c] = from_f32<T>(act ? conv_silu(acc) : acc);
     return;
   }
   const int b = item - n_rows;
@@ -222,7 +226,7 @@ __global__ void short_conv_kernel(const T* __restrict__ x, const float* __restri
   T* st = hist > 0 ? state + (static_cast<size_t>(slots[b]) * hist) * C + c : nullptr;
   // input at local index idx (negative: from the slot)
   auto input = [&](int idx) -> float {
-    if (idx >= 0) return to_f32(x[static_cast<size_t>(q0 + idx) * C + c]);
+    if (idx >= 0) return to_f32(x[static_cast<size_t>(q0 + idx) * ldx + c]);
     return fresh ? 0.f : to_f32(st[static_cast<size_t>(idx + hist) * C]);
   };
   const float* wc = w + static_cast<size_t>(c) * taps;
@@ -230,7 +234,7 @@ __global__ void short_conv_kernel(const T* __restrict__ x, const float* __restri
   for (int i = 0; i < head; ++i) {
     float acc = residual ? input(i) : 0.f;
     for (int j = 0; j < taps; ++j) acc += wc[j] * input(i - hist + j);
-    out[static_cast<size_t>(q0 + i) * C + c] = from_f32<T>(acc);
+    out[static_cast<size_t>(q0 + i) * C + c] = from_f32<T>(act ? conv_silu(acc) : acc);
   }
   // slot entry k becomes the input at local index n - hist + k; rising k reads
   // entries k + n > k only, never one already rewritten
@@ -247,7 +251,7 @@ template <typename T>
 __global__ void short_conv_vec_kernel(const T* __restrict__ x, const float* __restrict__ w, T* __restrict__ state,
                                       const int32_t* __restrict__ q_start, const int32_t* __restrict__ positions,
                                       const int32_t* __restrict__ slots, T* __restrict__ out, int n_rows, int B, int C,
-                                      int taps, int residual) {
+                                      int taps, int residual, int ldx, int act) {
   constexpr int VEC = 16 / sizeof(T);
   typedef T VecT __attribute__((ext_vector_type(VEC)));
   const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
@@ -259,7 +263,7 @@ __global__ void short_conv_vec_kernel(const T* __restrict__ x, const float* __re
   auto store = [&](T* p, const float (&v)[VEC]) {
     VecT o;
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) o[e] = from_f32<T>(v[e]);
+    for (int e = 0; e < VEC; ++e) o[e] = from_f32<T>(act ? conv_silu(v[e]) : v[e]);
     *reinterpret_cast<VecT*>(p) = o;
   };
   float wr[VEC][kConvTaps];   // this thread's channels x taps
@@ -284,7 +288,7 @@ __global__ void short_conv_vec_kernel(const T* __restrict__ x, const float* __re
 #pragma unroll
       for (int j = 0; j < kConvTaps; ++j) {
         if (j < taps) {
-          const VecT v = load(x + static_cast<size_t>(row - hist + j) * C + c);
+          const VecT v = load(x + static_cast<size_t>(row - hist + j) * ldx + c);
 #pragma unroll
           for (int e = 0; e < VEC; ++e) {
             acc[e] += wr[e][j] * to_f32(v[e]);
@@ -302,7 +306,7 @@ __global__ void short_conv_vec_kernel(const T* __restrict__ x, const float* __re
   const bool fresh = positions[q0] == 0;
   T* st = hist > 0 ? state + (static_cast<size_t>(slots[b]) * hist) * C + c : nullptr;
   auto input = [&](int idx) -> VecT {   // input at local index idx (negative: from the slot)
-    if (idx >= 0) return load(x + static_cast<size_t>(q0 + idx) * C + c);
+    if (idx >= 0) return load(x + static_cast<size_t>(q0 + idx) * ldx + c);
     VecT z;
 #pragma unroll
     for (int e = 0; e < VEC; ++e) z[e] = from_f32<T>(0.f);
@@ -722,18 +726,19 @@ int lyp_add_row(float* h, const float* v, int n_rows, int H, hipStream_t stream)
   return 0;
 }
 
-// x, out [n_rows, C] and state [slots, taps - 1, C] of dtype; w float [C, taps].
+// x [n_rows, >= C] (rows ldx apart), out [n_rows, C] and state [slots, taps - 1, C] of dtype; w float [C, taps].
 int lyp_short_conv(const void* x, const float* w, void* state, const int32_t* q_start, const int32_t* positions,
                    const int32_t* slots, void* out, int dtype, int n_rows, int B, int C, int taps, int residual,
-                   hipStream_t stream) {
+                   int ldx, int act, hipStream_t stream) {
   LYP_REQUIRE(n_rows >= 0 && B > 0 && C > 0 && taps >= 1, "short_conv: bad sizes rows=%d B=%d C=%d taps=%d", n_rows, B,
               C, taps);
   LYP_REQUIRE(taps == 1 || state != nullptr, "short_conv: %d taps need a state", taps);
   LYP_REQUIRE(x != out, "short_conv: in place is not possible");
+  LYP_REQUIRE(ldx >= C && (act == 0 || act == 1), "short_conv: input rows %d apart for %d channels, activation %d", ldx, C, act);
   if (n_rows == 0) return 0;
   const int vlen = dtype == kF32 ? 4 : 8;
   auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
-  if ((dtype == kF32 || dtype == kBF16) && C % vlen == 0 && taps <= kConvTaps && aligned(x) && aligned(out) &&
+  if ((dtype == kF32 || dtype == kBF16) && C % vlen == 0 && ldx % vlen == 0 && taps <= kConvTaps && aligned(x) && aligned(out) &&
       aligned(state)) {
     const int units = C / vlen;
     const int vt = units >= 256 ? 256 : 64 * ((units + 63) / 64);
@@ -741,11 +746,11 @@ int lyp_short_conv(const void* x, const float* w, void* state, const int32_t* q_
     if (dtype == kF32)
       short_conv_vec_kernel<float><<<vgrid, vt, 0, stream>>>(static_cast<const float*>(x), w,
                                                              static_cast<float*>(state), q_start, positions, slots,
-                                                             static_cast<float*>(out), n_rows, B, C, taps, residual);
+                                                             static_cast<float*>(out), n_rows, B, C, taps, residual, ldx, act);
     else
       short_conv_vec_kernel<bf16_t><<<vgrid, vt, 0, stream>>>(static_cast<const bf16_t*>(x), w,
                                                               static_cast<bf16_t*>(state), q_start, positions, slots,
-                                                              static_cast<bf16_t*>(out), n_rows, B, C, taps, residual);
+                                                              static_cast<bf16_t*>(out), n_rows, B, C, taps, residual, ldx, act);
     LYP_LAUNCH_CHECK("short_conv");
     return 0;
   }
@@ -754,11 +759,11 @@ int lyp_short_conv(const void* x, const float* w, void* state, const int32_t* q_
   if (dtype == kF32)
     short_conv_kernel<float><<<grid, threads, 0, stream>>>(static_cast<const float*>(x), w, static_cast<float*>(state),
                                                            q_start, positions, slots, static_cast<float*>(out), n_rows,
-                                                           B, C, taps, residual);
+                                                           B, C, taps, residual, ldx, act);
   else if (dtype == kBF16)
     short_conv_kernel<bf16_t><<<grid, threads, 0, stream>>>(static_cast<const bf16_t*>(x), w,
                                                             static_cast<bf16_t*>(state), q_start, positions, slots,
-                                                            static_cast<bf16_t*>(out), n_rows, B, C, taps, residual);
+                                                            static_cast<bf16_t*>(out), n_rows, B, C, taps, residual, ldx, act);
   else
     LYP_REQUIRE(false, "short_conv: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("short_conv");

@@ -11,7 +11,7 @@ from __future__ import annotations
 import ctypes
 import math
 import os
-from ctypes import c_float, c_int, c_longlong, c_void_p
+from ctypes import c_double, c_float, c_int, c_longlong, c_void_p
 
 import torch
 
@@ -93,7 +93,7 @@ def core() -> ctypes.CDLL:
                                         c_void_p, c_int, c_void_p]
         lib.lyp_add_row.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p]
         lib.lyp_short_conv.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                                       c_int, c_int, c_int, c_int, c_int, c_void_p]
+                                       c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]
         lib.lyp_activation.argtypes = [c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p, c_void_p]
         lib.lyp_mingru_scan.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int, c_int, c_int, c_void_p]
@@ -126,10 +126,31 @@ def core() -> ctypes.CDLL:
                                      c_void_p, c_void_p]
         lib.lyp_moe_gemm.argtypes = [c_void_p, c_int, c_void_p, c_longlong, c_int, c_void_p, c_int, c_int, c_int,
                                      c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
-                                     c_float, c_float, c_void_p]
+                                     c_float, c_float, c_int, c_void_p]
         lib.lyp_glu_clamped.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_float, c_void_p]
         lib.lyp_moe_combine.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                         c_int, c_void_p]
+        lib.lyp_group_rmsnorm.argtypes = [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_void_p, c_int,
+                                          c_void_p, c_int, c_int, c_int, c_float, c_void_p]
+        lib.lyp_add_sinusoid.argtypes = [c_void_p, c_void_p, c_int, c_int, c_double, c_void_p]
+        lib.lyp_glu_act.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
+        lib.lyp_gate_mul.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]
+        lib.lyp_weighted_sum.argtypes = [c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_float, c_void_p, c_int,
+                                         c_int, c_void_p]
+        lib.lyp_qkv_bias_temper_kv.argtypes = [c_void_p, c_int, c_void_p, c_void_p, c_float, c_int, c_void_p, c_void_p,
+                                               c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                               c_void_p]
+        lib.lyp_linear_scan_lanes.argtypes = [c_int]
+        lib.lyp_linear_scan.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int,
+                                        c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                        c_float, c_void_p]
+        lib.lyp_head_norm_gate.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
+                                           c_int, c_float, c_int, c_void_p]
+        lib.lyp_lowrank_up.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                       c_void_p]
+        lib.lyp_moe_route_grouped.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                              c_int, c_int, c_float, c_void_p, c_void_p, c_void_p]
         _core = lib
     return _core
 
@@ -933,12 +954,22 @@ def add_row(h: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
     return h
 
 
+def _rows_view(t: torch.Tensor, what: str) -> None:
+    """A 2-d GPU tensor whose rows' values are neighbours (a column range of a wider tensor is fine)."""
+    if t is None or not t.is_cuda or t.dim() != 2 or t.stride(1) != 1 or t.stride(0) < t.shape[1]:
+        raise KernelError(f"{what}: a 2-d GPU tensor whose rows' values are neighbours, not "
+                          f"{None if t is None else (tuple(t.shape), t.stride(), str(t.device))}")
+
+
 def short_conv(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor | None, q_start: torch.Tensor,
-               positions: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, B: int, residual: bool = True):
+               positions: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, B: int, residual: bool = True,
+               silu: bool = False):
     """out = (x +) the causal filter of x over time, channel by channel, request by request:
     w float [C, taps]; ``state`` [slots, taps - 1, C] of x's type holds every request's last inputs
-    from earlier steps (not read for a request at position 0) and is brought up to date."""
-    _dev(x, w, state, q_start, positions, slots, out)
+    from earlier steps (not read for a request at position 0) and is brought up to date.  x may be a
+    column range of a wider tensor; ``silu``: the result passes x * sigmoid(x)."""
+    _rows_view(x, "short_conv")
+    _dev(w, state, q_start, positions, slots, out)
     _f32(w)
     T, C = x.shape
     taps = w.shape[1]
@@ -950,7 +981,7 @@ def short_conv(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor | None, q_s
         raise KernelError("short_conv: the step's tables do not fit its rows and requests")
     lib = core()
     _check(lib.lyp_short_conv(_p(x), _p(w), _p(state), _p(q_start), _p(positions), _p(slots), _p(out), _code(x.dtype),
-                              T, B, C, taps, int(residual), _stream()), lib)
+                              T, B, C, taps, int(residual), x.stride(0), int(silu), _stream()), lib)
     return out
 
 
@@ -1435,21 +1466,24 @@ def moe_sort(idx: torch.Tensor, num_experts: int) -> MoePlan:
 
 
 def moe_gemm(a: torch.Tensor, w: torch.Tensor, plan: MoePlan, *, gated: bool, limit: float = 0.0,
-             alpha: float = 0.0) -> torch.Tensor:
+             alpha: float = 0.0, gather: bool = False, relu2: bool = False) -> torch.Tensor:
     """One product per expert over the rows sorted to it.  gated: a [T, K] (rows gathered by token),
     w [E, 2 N, K] (an expert's gate rows, then its up rows) -> [pairs, N], the gated activation of
-    ``glu_clamped`` applied.  Otherwise a [pairs, K] in sorted order, w [E, N, K] -> [pairs, N]."""
+    ``glu_clamped`` applied.  Otherwise a [pairs, K] in sorted order, w [E, N, K] -> [pairs, N]; with
+    ``gather`` a is [T, K] and gathered by token as for a gated product, with ``relu2`` the result
+    is max(y, 0)^2."""
     _dev(a, w)
     E, rows, K = w.shape
     N = rows // 2 if gated else rows
-    if a.dtype != w.dtype or a.shape[1] != K or E != plan.E or (not gated and a.shape[0] != plan.pairs):
+    if a.dtype != w.dtype or a.shape[1] != K or E != plan.E or (not gated and not gather and a.shape[0] != plan.pairs) \
+            or (gated and (gather or relu2)):
         raise KernelError(f"moe_gemm: a {tuple(a.shape)} {a.dtype}, w {tuple(w.shape)} {w.dtype}, {plan.pairs} pairs")
     out = torch.empty((plan.pairs, N), dtype=a.dtype, device=a.device)
     lib = core()
     _check(lib.lyp_moe_gemm(_p(a), a.stride(0), _p(w), w.stride(0), w.stride(1), _p(out), out.stride(0), _code(a.dtype),
                             int(gated), _p(plan.tile_expert), _p(plan.tile_row0), _p(plan.n_tiles), plan.most_tiles,
                             plan.tile_rows, _p(plan.expert_off), _p(plan.sorted_pair), plan.top, N, K, float(limit),
-                            float(alpha), _stream()), lib)
+                            float(alpha), int(gather) | 2 * int(relu2), _stream()), lib)
     return out
 
 
@@ -1470,6 +1504,232 @@ def moe_combine(y: torch.Tensor, plan: MoePlan, weights: torch.Tensor, rows: int
     _check(lib.lyp_moe_combine(_p(y), _p(plan.place_of), _p(weights), plan.top, _p(addend), _p(shared), _p(out),
                                _code(y.dtype), rows, H, _stream()), lib)
     return out
+
+
+def moe_route_grouped(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor | None, top: int, groups: int,
+                      keep: int, scale: float):
+    """Sigmoid scores s = sigmoid(x @ router.T) in 32-bit (x [T, K] activations, router [E, K] float); the
+    choice goes by s + correction among the experts of the ``keep`` best of ``groups`` equal groups of
+    neighbours (a group's score: the sum of its two largest choice scores), the weights are the chosen
+    experts' s over their sum, times ``scale``.  -> (experts int32 [T, top], weights float [T, top])."""
+    _rows_view(x, "moe_route_grouped")
+    _dev(router, correction)
+    _f32(router, correction)
+    T, K = x.shape
+    E = router.shape[0]
+    if router.shape[1] != K or (correction is not None and correction.numel() != E):
+        raise KernelError(f"moe_route_grouped: x {tuple(x.shape)}, router {tuple(router.shape)}")
+    idx = torch.empty((T, top), dtype=torch.int32, device=x.device)
+    wgt = torch.empty((T, top), dtype=torch.float32, device=x.device)
+    lib = core()
+    _check(lib.lyp_moe_route_grouped(_p(x), x.stride(0), _code(x.dtype), _p(router), _p(correction), T, E, K, top,
+                                     int(groups), int(keep), float(scale), _p(idx), _p(wgt), _stream()), lib)
+    return idx, wgt
+
+
+# ------------------------------------- grouped norms, scaled branches, gates, recurrences
+class ScaledBranch:
+    """A branch's output that joins the residual stream times a vector: h += y * scale.  ``y`` is
+    [T, H] in the activations' type or float, or float partial sums [S, T, H]; ``scale`` float [H].
+    A norm with ``takes_scaled`` does the sum in its own kernel; ``join(h)`` does it alone."""
+
+    def __init__(self, y: torch.Tensor, scale: torch.Tensor):
+        if isinstance(y, PendingLinear):
+            y = y.run()
+        self.y, self.scale = y, scale
+        self.shape = y.shape
+
+    def join(self, h: torch.Tensor) -> None:
+        """Carry the sum out on h; nothing is left to add (returns None)."""
+        group_rmsnorm(h, None, 1, 0.0, None, delta=self.y, scale=self.scale)
+        return None
+
+
+def group_rmsnorm(h: torch.Tensor, weight: torch.Tensor | None, groups: int, eps: float, out: torch.Tensor | None,
+                  delta: torch.Tensor | None = None, scale: torch.Tensor | None = None,
+                  rows: torch.Tensor | None = None):
+    """h += scale * delta on the float residual stream (``delta`` [T, H] in the activations' type or
+    float, or float partial sums [S, T, H]; ``scale`` float [H] or None), then out = every one of
+    ``groups`` equal consecutive parts of a row over its own root mean square, the row times
+    ``weight`` (float).  ``rows`` picks the rows to norm and leaves h alone; out None: the sum only."""
+    _dev(h, weight, out, delta, scale, rows)
+    _f32(h, weight, scale)
+    T, H = h.shape
+    n = T if rows is None else rows.numel()
+    parts, stride = 0, 0
+    if delta is not None:
+        if delta.dim() == 3:
+            if delta.dtype != torch.float32 or tuple(delta.shape[1:]) != (T, H):
+                raise KernelError(f"group_rmsnorm: partial sums {tuple(delta.shape)} {delta.dtype} against h {tuple(h.shape)}")
+            parts, stride = delta.shape[0], T * H
+        elif tuple(delta.shape) != (T, H):
+            raise KernelError(f"group_rmsnorm: delta {tuple(delta.shape)} against h {tuple(h.shape)}")
+    if (scale is not None and scale.numel() != H) or (out is not None and (weight is None or weight.numel() != H or
+                                                                           tuple(out.shape) != (n, H))):
+        raise KernelError("group_rmsnorm: scale and weight have one value per feature, the output one row per normed row")
+    if rows is not None and (rows.dtype != torch.int32 or out is None):
+        raise KernelError("group_rmsnorm: rows are int32 and only picked for an output")
+    lib = core()
+    _check(lib.lyp_group_rmsnorm(_p(h), _p(delta), _code(delta.dtype) if delta is not None else 0, parts, stride,
+                                 _p(scale), _p(weight), _p(out), _code(out.dtype) if out is not None else 0, _p(rows), n,
+                                 H, int(groups), float(eps), _stream()), lib)
+    return out
+
+
+def add_sinusoid(h: torch.Tensor, positions: torch.Tensor, base: float) -> torch.Tensor:
+    """h[t, 2i] += sin(p_t * base^(-2i/H)), h[t, 2i+1] += cos(the same) on a float tensor [T, H]."""
+    _dev(h, positions)
+    _f32(h)
+    if positions.dtype != torch.int32 or positions.numel() != h.shape[0]:
+        raise KernelError("add_sinusoid: one int32 position per row")
+    lib = core()
+    _check(lib.lyp_add_sinusoid(_p(h), _p(positions), h.shape[0], h.shape[1], float(base), _stream()), lib)
+    return h
+
+
+GLU_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def glu_act(gate_up: torch.Tensor, activation: str) -> torch.Tensor:
+    """[T, 2 I] (a row's gates, then its ups) -> act(gate) * up [T, I]."""
+    _dev(gate_up)
+    if activation not in GLU_ACTIVATIONS or gate_up.dim() != 2 or gate_up.shape[1] % 2:
+        raise KernelError(f"glu_act: {activation!r} on {tuple(gate_up.shape)}")
+    T, I = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((T, I), dtype=gate_up.dtype, device=gate_up.device)
+    lib = core()
+    _check(lib.lyp_glu_act(_p(gate_up), _p(out), _code(gate_up.dtype), T, I, GLU_ACTIVATIONS[activation], _stream()), lib)
+    return out
+
+
+GATES = {"sigmoid": 0, "silu": 1}
+
+
+def gate_mul(x: torch.Tensor, gate: torch.Tensor, kind: str) -> torch.Tensor:
+    """x *= sigmoid(gate) or silu(gate), in place: x [T, N] activations, gate [T, N] float or of x's
+    type, possibly a column range of a wider tensor."""
+    _dev(x)
+    _rows_view(gate, "gate_mul")
+    if kind not in GATES or gate.shape != x.shape or gate.dtype not in (torch.float32, x.dtype):
+        raise KernelError(f"gate_mul: {kind!r}, x {tuple(x.shape)} {x.dtype}, gate {tuple(gate.shape)} {gate.dtype}")
+    lib = core()
+    _check(lib.lyp_gate_mul(_p(x), _code(x.dtype), _p(gate), gate.stride(0), _code(gate.dtype), x.shape[0], x.shape[1],
+                            GATES[kind], _stream()), lib)
+    return x
+
+
+def weighted_sum(a: torch.Tensor, sa: float, b: torch.Tensor, sb: float, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """float [1, T, H] (one slice of partial sums for the residual stream) = sa * (a + bias) + sb * b."""
+    _dev(a, b, bias)
+    _f32(bias)
+    if a.shape != b.shape or a.dim() != 2 or (bias is not None and bias.numel() != a.shape[1]):
+        raise KernelError(f"weighted_sum: {tuple(a.shape)} and {tuple(b.shape)}")
+    T, H = a.shape
+    out = torch.empty((1, T, H), dtype=torch.float32, device=a.device)
+    lib = core()
+    _check(lib.lyp_weighted_sum(_p(a), _code(a.dtype), _p(bias), float(sa), _p(b), _code(b.dtype), float(sb), _p(out), T, H,
+                                _stream()), lib)
+    return out
+
+
+def qkv_bias_temper_kv(pre: torch.Tensor, bias: torch.Tensor | None, positions: torch.Tensor, coef: float, every: int,
+                       slots: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, dtype: torch.dtype, *,
+                       num_heads: int, num_kv_heads: int, dim: int, vdim: int, page_size: int) -> torch.Tensor:
+    """From a float projection pre [T, >= (H + G) dim + G vdim] (queries, keys, values side by side):
+    bias added, queries times 1 + coef * ln(floor((p + 1) / every) + 1) returned as [T, H dim] of
+    ``dtype``, keys and values into the tokens' page slots (keys [pages, G, page, dim], values
+    [pages, G, vdim, page])."""
+    _rows_view(pre, "qkv_bias_temper_kv")
+    _dev(bias, positions, slots, kpool, vpool)
+    _f32(pre, bias)
+    T = pre.shape[0]
+    H, G = num_heads, num_kv_heads
+    n = (H + G) * dim + G * vdim
+    n_pages = kpool.shape[0]
+    if pre.shape[1] < n or (bias is not None and bias.numel() != n) or positions.numel() != T or slots.numel() != T or \
+            positions.dtype != torch.int32 or slots.dtype != torch.int32 or every < 1 or \
+            tuple(kpool.shape) != (n_pages, G, page_size, dim) or tuple(vpool.shape) != (n_pages, G, vdim, page_size) or \
+            kpool.dtype != dtype or vpool.dtype != dtype:
+        raise KernelError(f"qkv_bias_temper_kv: pre {tuple(pre.shape)}, pools {tuple(kpool.shape)} / {tuple(vpool.shape)} "
+                          f"{kpool.dtype} for {H}+{G} heads of {dim}/{vdim}, pages of {page_size}, dtype {dtype}")
+    q = torch.empty((T, H * dim), dtype=dtype, device=pre.device)
+    lib = core()
+    _check(lib.lyp_qkv_bias_temper_kv(_p(pre), pre.stride(0), _p(bias), _p(positions), float(coef), int(every), _p(slots),
+                                      _p(q), _p(kpool), _p(vpool), _code(dtype), T, H, G, dim, vdim, page_size,
+                                      _stream()), lib)
+    return q
+
+
+LINEAR_SCAN_MAX_DIM = 256    # key channels a head of ``linear_scan`` may have
+
+
+def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor, zbias: torch.Tensor | None,
+                coef: torch.Tensor, sign: float, state: torch.Tensor, q_start: torch.Tensor, positions: torch.Tensor,
+                slots: torch.Tensor, out: torch.Tensor, B: int, *, num_heads: int, num_kv_heads: int, dim: int,
+                vdim: int, beta: torch.Tensor | None = None, unit: bool = False, q_scale: float = 1.0) -> torch.Tensor:
+    """The recurrence with a matrix state per head over the step's rows, request by request, in order:
+    S <- diag(g) S (+ the delta rule's correction when ``beta`` is given) + k v^T, out = S^T q, with
+    g = exp(-coef[head] * softplus(sign * (z + zbias))).  q, k [T, G dim] and v [T, H vdim] are
+    activations (column ranges of wider tensors are fine), z float [T, H dim], beta [T, H] activations
+    (before its sigmoid), state float [slots, H, vdim, dim] (a head's matrix transposed), out float
+    [T, H vdim].  ``unit``: q and k become unit vectors per head first; q is multiplied by ``q_scale``."""
+    for t, what in ((q, "q"), (k, "k"), (v, "v"), (z, "z")) + (((beta, "beta"),) if beta is not None else ()):
+        _rows_view(t, f"linear_scan {what}")
+    _dev(zbias, coef, state, q_start, positions, slots, out)
+    _f32(z, zbias, coef, state, out)
+    T = out.shape[0]
+    H, G = num_heads, num_kv_heads
+    if q.dtype != k.dtype or q.dtype != v.dtype or (beta is not None and beta.dtype != q.dtype) or \
+            q.shape[0] != T or k.shape[0] != T or v.shape[0] != T or z.shape[0] != T or \
+            q.shape[1] != G * dim or k.shape[1] != G * dim or v.shape[1] != H * vdim or z.shape[1] != H * dim or \
+            (beta is not None and tuple(beta.shape) != (T, H)) or tuple(out.shape) != (T, H * vdim) or \
+            tuple(state.shape[1:]) != (H, vdim, dim) or coef.numel() != H or \
+            (zbias is not None and zbias.numel() != H * dim) or q_start.numel() != B + 1 or slots.numel() != B or \
+            positions.numel() != T:
+        raise KernelError(f"linear_scan: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}, z {tuple(z.shape)}, "
+                          f"state {tuple(state.shape)}, out {tuple(out.shape)} for {H}/{G} heads of {dim}/{vdim}")
+    lib = core()
+    _check(lib.lyp_linear_scan(_p(q), q.stride(0), _p(k), k.stride(0), _p(v), v.stride(0), _code(q.dtype), _p(z),
+                               z.stride(0), _p(zbias), _p(coef), float(sign), _p(beta),
+                               beta.stride(0) if beta is not None else 0, _p(state), _p(q_start), _p(positions), _p(slots),
+                               _p(out), out.stride(0), B, H, G, dim, vdim, int(beta is not None), int(unit),
+                               float(q_scale), _stream()), lib)
+    return out
+
+
+def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, kind: str, eps: float,
+                   dtype: torch.dtype, *, num_heads: int, vdim: int) -> torch.Tensor:
+    """o float [T, H vdim]: every head divided by its root mean square over vdim, times ``weight``
+    (float [vdim], shared by the heads), times sigmoid or silu of ``gate`` [T, H vdim] (float or of
+    ``dtype``, possibly a column range); -> [T, H vdim] of ``dtype``."""
+    _dev(o, weight)
+    _rows_view(gate, "head_norm_gate")
+    _f32(o, weight)
+    T = o.shape[0]
+    if kind not in GATES or tuple(o.shape) != (T, num_heads * vdim) or gate.shape != o.shape or weight.numel() != vdim or \
+            gate.dtype not in (torch.float32, dtype):
+        raise KernelError(f"head_norm_gate: o {tuple(o.shape)}, gate {tuple(gate.shape)} {gate.dtype}, {num_heads} heads of {vdim}")
+    out = torch.empty((T, num_heads * vdim), dtype=dtype, device=o.device)
+    lib = core()
+    _check(lib.lyp_head_norm_gate(_p(o), _p(weight), _p(gate), gate.stride(0), _code(gate.dtype), _p(out), _code(dtype), T,
+                                  num_heads, vdim, float(eps), GATES[kind], _stream()), lib)
+    return out
+
+
+def lowrank_up(mid: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """float [T, N] = mid @ w.T (+ bias) in 32-bit: mid [T, R] activations (a column range is fine), w float [N, R]."""
+    _rows_view(mid, "lowrank_up")
+    _dev(w, bias)
+    _f32(w, bias)
+    T, R = mid.shape
+    N = w.shape[0]
+    if w.shape[1] != R or (bias is not None and bias.numel() != N):
+        raise KernelError(f"lowrank_up: mid {tuple(mid.shape)}, w {tuple(w.shape)}")
+    out = torch.empty((T, N), dtype=torch.float32, device=mid.device)
+    lib = core()
+    _check(lib.lyp_lowrank_up(_p(mid), mid.stride(0), _code(mid.dtype), _p(w), _p(bias), _p(out), T, N, R, _stream()), lib)
+    return out
+
 
 
 # -------------------------------------------------------------------- sampling

@@ -183,6 +183,8 @@ class DecoderModel(Part):
         first = self.embedding.forward(ctx, ctx.token_ids) if any(c.reinject for c in self.schedule) else None
         delta = None
         for call, cache in zip(self.schedule, caches):
+            if isinstance(delta, ops.ScaledBranch) and (call.reinject or call.shift is not None):
+                delta = delta.join(h)
             if call.reinject:
                 if isinstance(delta, ops.JoiningBranch):
                     delta = delta.join(h)
@@ -196,6 +198,8 @@ class DecoderModel(Part):
         if isinstance(delta, ops.PendingLinear) and not getattr(self.final_norm, "can_defer", False):
             delta = delta.run()
         if isinstance(delta, ops.JoiningBranch) and not getattr(self.final_norm, "joins_branches", False):
+            delta = delta.join(h)
+        if isinstance(delta, ops.ScaledBranch) and not getattr(self.final_norm, "takes_scaled", False):
             delta = delta.join(h)
         x = self.final_norm.forward(ctx, h, delta, rows=ctx.logit_rows)
         out = self.head.forward(ctx, x)

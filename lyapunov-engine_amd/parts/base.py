@@ -32,7 +32,24 @@ import torch
 @dataclass(frozen=True)
 class WeightSource:
     name: str              # tensor name in the file, relative to the part's prefix
-    shape: tuple
+    shape: tuple           # a negative entry -n: the file decides this size (``free_size``); n when values are made up
+
+
+def free_size(made_up: int) -> int:
+    """An entry of a ``WeightSource.shape`` whose size the file's tensor decides (a projection's
+    inner rank that no configuration names); ``made_up`` is the size random weights get."""
+    if made_up < 1:
+        raise ValueError(f"a made-up size is at least 1, not {made_up}")
+    return -int(made_up)
+
+
+def shape_fits(got: tuple, want: tuple) -> bool:
+    """Whether a file's tensor of shape ``got`` is what a ``WeightSource`` of shape ``want`` asks for."""
+    return len(got) == len(want) and all(w < 0 or int(g) == int(w) for g, w in zip(got, want))
+
+
+def made_up_shape(want: tuple) -> tuple:
+    return tuple(abs(int(w)) for w in want)
 
 
 @dataclass(frozen=True)
@@ -344,6 +361,13 @@ class Mixer(Part):
     def state_spec(self) -> Optional[StateSpec]:
         return None
 
+    def further_states(self) -> dict:
+        """More state per live request than the one slot tensor of ``state_spec`` (the last inputs
+        of a short convolution beside a recurrence's summary, ...): name -> StateSpec.  The layer's
+        block asks for them with its own (``Block.state_specs``); the tensors reach ``forward`` as
+        ``cache.states["mixer." + name]``."""
+        return {}
+
     def forward(self, ctx: StepContext, x: torch.Tensor, cache: LayerCache) -> torch.Tensor:
         raise NotImplementedError
 
@@ -388,8 +412,9 @@ class Block(Part):
     def state_specs(self) -> dict:
         """State per live request that parts of the arrangement other than the
         mixer keep (an input filter's last inputs, ...): name -> StateSpec; the
-        tensors reach ``forward`` as ``cache.states[name]``."""
-        return {}
+        tensors reach ``forward`` as ``cache.states[name]``.  The mixer's further states are among
+        them under "mixer.<name>"."""
+        return {"mixer." + name: spec for name, spec in self.mixer.further_states().items()}
 
     def forward(self, ctx: StepContext, h: torch.Tensor, delta: Optional[torch.Tensor],
                 cache: LayerCache) -> tuple:
@@ -398,7 +423,7 @@ class Block(Part):
 
 
 __all__ = [
-    "WeightSource", "WeightSpec", "Part", "PagedSpec", "PageTensor", "SLOT", "StateSpec", "GroupView", "LayerCache", "StepContext",
+    "WeightSource", "WeightSpec", "free_size", "shape_fits", "made_up_shape", "Part", "PagedSpec", "PageTensor", "SLOT", "StateSpec", "GroupView", "LayerCache", "StepContext",
     "StepBatch", "StepPlan", "StepPlanner", "FixedStep",
     "Norm", "PositionEncoding", "Mixer", "FeedForward", "InputFilter", "StreamShift", "Block", "Logits", "Any",
 ]

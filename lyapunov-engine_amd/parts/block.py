@@ -13,7 +13,7 @@ import torch
 from ..config.registry import BLOCKS, FEED_FORWARDS, FILTERS, MIXERS, NORMS
 from ..config.specs import LayerSpec
 from ..kernels import ops
-from .base import Block, LayerCache, StepContext
+from .base import Block, LayerCache, StepContext, WeightSource, WeightSpec
 
 
 @BLOCKS.register("prenorm")
@@ -74,8 +74,11 @@ class SandwichBlock(Block):
         return out
 
     def state_specs(self):
+        out = super().state_specs()
         st = self.filter.state_spec() if self.filter is not None else None
-        return {"filter": st} if st is not None else {}
+        if st is not None:
+            out["filter"] = st
+        return out
 
     def forward(self, ctx: StepContext, h, delta, cache: LayerCache):
         conv = None
@@ -94,6 +97,73 @@ class SandwichBlock(Block):
             return h, branch
         x = self.norm2.forward(ctx, h, branch)
         return h, self.norm2_out.branch(self.ffn.forward(ctx, x), self.mult)
+
+
+@BLOCKS.register("prenorm_scaled")
+class ScaledPreNormBlock(Block):
+    """The pre-norm arrangement with a learned vector on what each branch adds, and optionally a
+    filter over time on what the mixer reads:
+
+        h += s1 * mixer(filter(norm1(h)));  h += s2 * ffn(norm2(h))
+
+    s1 and s2 are tensors of the layer itself (``names["scale1"]``, ``names["scale2"]``); the filter
+    comes from ``LayerSpec.extra["filter"]``.  The feed-forward branch may be absent.  A branch's
+    product with its vector and the sum are carried out by the norm that follows (one with
+    ``takes_scaled``, through an ``ops.ScaledBranch``); the block returns its last branch still to
+    be added."""
+
+    def __init__(self, spec: LayerSpec):
+        self.names = dict(spec.names)
+        self.norm1 = NORMS.build(spec.norm1)
+        self.mixer = MIXERS.build(spec.mixer)
+        self.filter = FILTERS.build(spec.extra["filter"]) if "filter" in spec.extra else None
+        self.ffn = FEED_FORWARDS.build(spec.ffn) if spec.ffn is not None else None
+        self.norm2 = NORMS.build(spec.norm2) if self.ffn is not None else None
+        self.hidden_size = int(spec.params["hidden_size"])
+        self.scale1 = self.scale2 = None
+        self.scale1_f = self.scale2_f = None
+        unknown = set(spec.extra) - {"filter"}
+        if unknown:
+            raise ValueError(f"the scaled pre-norm arrangement has no parts {sorted(unknown)}")
+
+    def weight_specs(self):
+        n, shape = self.names, (self.hidden_size,)
+        specs = [WeightSpec("scale1", (WeightSource(n["scale1"], shape),), init="ones")]
+        if self.ffn is not None:
+            specs.append(WeightSpec("scale2", (WeightSource(n["scale2"], shape),), init="ones"))
+        return specs
+
+    def children(self):
+        n = self.names
+        out = {n["norm1"]: self.norm1, n["mixer"]: self.mixer}
+        if self.filter is not None:
+            out[n["filter"]] = self.filter
+        if self.ffn is not None:
+            out.update({n["norm2"]: self.norm2, n["ffn"]: self.ffn})
+        return out
+
+    def materialize(self, device, dtype):
+        super().materialize(device, dtype)
+        self.scale1_f = self.scale1.float().contiguous()
+        if self.scale2 is not None:
+            self.scale2_f = self.scale2.float().contiguous()
+
+    def state_specs(self):
+        out = super().state_specs()
+        st = self.filter.state_spec() if self.filter is not None else None
+        if st is not None:
+            out["filter"] = st
+        return out
+
+    def forward(self, ctx: StepContext, h, delta, cache: LayerCache):
+        x = normed(self.norm1, None, ctx, h, delta)
+        if self.filter is not None:
+            x = self.filter.forward(ctx, x, cache.states.get("filter"))
+        branch = ops.ScaledBranch(self.mixer.forward(ctx, x, cache), self.scale1_f)
+        if self.ffn is None:
+            return h, branch
+        x = normed(self.norm2, None, ctx, h, branch)
+        return h, ops.ScaledBranch(self.ffn.forward(ctx, x), self.scale2_f)
 
 
 @BLOCKS.register("parallel")
@@ -138,6 +208,8 @@ def normed(norm, consumer, ctx: StepContext, h, delta):
     a norm that does not know of pending products gets the product itself, and
     one that does not know of joining branches finds the branch joined."""
     if isinstance(delta, ops.JoiningBranch) and not getattr(norm, "joins_branches", False):
+        delta = delta.join(h)
+    if isinstance(delta, ops.ScaledBranch) and not getattr(norm, "takes_scaled", False):
         delta = delta.join(h)
     if getattr(norm, "can_defer", False):
         return norm.forward(ctx, h, delta, lazy=getattr(consumer, "takes_pending_norm", False))

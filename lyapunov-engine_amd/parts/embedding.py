@@ -14,7 +14,7 @@ from typing import Optional
 
 import torch
 
-from ..config.registry import EMBEDDINGS, HEADS, STREAM_SHIFTS
+from ..config.registry import EMBEDDINGS, HEADS, NORMS, STREAM_SHIFTS
 from ..kernels import ops
 from .base import Embedding, Head, Logits, StepContext, StreamShift, WeightSource, WeightSpec
 
@@ -34,6 +34,33 @@ class TokenEmbedding(Embedding):
     def forward(self, ctx: StepContext, token_ids: torch.Tensor) -> torch.Tensor:
         h = torch.empty((token_ids.numel(), self.hidden_size), dtype=torch.float32, device=ctx.device)
         return ops.embedding(token_ids, self.weight, h, self.scale)
+
+
+@EMBEDDINGS.register("lookup_sinusoid")
+class SinusoidEmbedding(TokenEmbedding):
+    """A looked-up row plus a position vector that is computed, not learned: entry 2i is
+    sin(p * base^(-2i / hidden)), entry 2i + 1 the cosine of the same angle (angles in 64-bit);
+    then, optionally, a norm of the sum (``norm``: a PartSpec of the NORMS registry, whose tensors
+    stand under ``norm_name`` after the embedding's prefix).  The normed rows are the residual
+    stream's first value, in 32-bit."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, scale: float = 1.0, tensor: str = "weight",
+                 base: float = 10000.0, norm=None, norm_name: str = "norm."):
+        super().__init__(vocab_size, hidden_size, scale, tensor)
+        if not base > 0:
+            raise ValueError(f"the sinusoid's base must be positive, not {base}")
+        self.base, self.norm_name = float(base), norm_name
+        self.norm = NORMS.build(norm) if norm is not None else None
+
+    def children(self):
+        return {self.norm_name: self.norm} if self.norm is not None else {}
+
+    def forward(self, ctx: StepContext, token_ids: torch.Tensor) -> torch.Tensor:
+        h = super().forward(ctx, token_ids)
+        ops.add_sinusoid(h, ctx.positions, self.base)
+        if self.norm is None:
+            return h
+        return self.norm.forward(ctx, h, out_dtype=torch.float32)
 
 
 @HEADS.register("linear")

@@ -47,3 +47,24 @@ class CausalShortConv(InputFilter):
         out = torch.empty_like(x)
         return ops.short_conv(x, self.weight_f, state, ctx.q_start, ctx.positions, ctx.state_slots, out, ctx.B,
                               residual=self.residual)
+
+
+@FILTERS.register("token_shift")
+class TokenShift(CausalShortConv):
+    """Every channel moves a learned part of the way towards the previous token's value:
+    out_t = x_t + (x_(t-1) - x_t) * mu, with x_(-1) = 0.  That is a convolution of two taps,
+    (mu, 1 - mu), without the residual; the previous token's input is the state."""
+
+    def __init__(self, channels: int, tensor: str = "weight"):
+        super().__init__(channels, taps=2, residual=False, tensor=tensor)
+        self.mix: Optional[torch.Tensor] = None
+
+    def weight_specs(self):
+        return [WeightSpec("mix", (WeightSource(self.tensor, (self.channels,)),))]
+
+    def materialize(self, device, dtype):
+        mu = self.mix.float()
+        self.weight_f = torch.stack([mu, 1.0 - mu], dim=1).contiguous()
+
+    def fused(self, ctx, state, width):
+        return None

@@ -1,0 +1,187 @@
+"""Mixers that carry a matrix per head instead of keys: a gated delta rule and
+gated linear attention, both with a decay per head and key channel.
+
+Per head, with S a matrix [dim x vdim] that starts at zero and lives in 32-bit
+in a state slot of the request:
+
+  "gated_delta_rule"
+    q, k (G heads of dim), v (H heads of vdim): projections, each through a short causal
+    convolution per channel and silu; q and k made unit vectors per head, q times dim^(-1/2);
+    query head h reads q/k head h // (H / G)
+    g = exp(-exp(A_h) * softplus(W_a2 (W_a1 x) + b_dt))      one decay per head and key channel
+    beta = sigmoid(W_b x)                                    one per head
+    S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+    y = W_o concat_h( o_h / rms(o_h) * w * sigmoid(W_g2 (W_g1 x)) )
+
+  "gated_linear_attention"
+    q = W_q x * dim^(-1/2), k = W_k x (H heads of dim), v = W_v x (H heads of vdim)
+    a = sigmoid(W_a2 (W_a1 x) + b)^(1 / tau)                 one decay per head and key channel
+    S <- diag(a) S + k v^T;  o = S^T q
+    y = W_o concat_h( o_h / rms(o_h) * w * silu(W_g x) )
+
+Everything that reads x is one product; the inner sizes of the low-rank pairs
+(W_a1, W_g1) are whatever the file's tensors have.  Decays, unit vectors, beta,
+the recurrence and the heads' norm are 32-bit (``ops.linear_scan``,
+``ops.head_norm_gate``); the state is kept transposed, [heads, vdim, dim].
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..config.registry import MIXERS
+from ..kernels import ops
+from .base import LayerCache, Mixer, StateSpec, StepContext, WeightSource, WeightSpec, free_size
+
+MADE_UP_RANK = 16   # inner size of the low-rank pairs when weights are made up
+
+
+def _scan_out(ctx: StepContext, width: int) -> torch.Tensor:
+    """The recurrence's float output; zeroed where a recorded prompt step has rows that belong to no request."""
+    make = torch.zeros if ctx.fixed is not None and ctx.fixed.tokens else torch.empty
+    return make((ctx.T, width), dtype=torch.float32, device=ctx.device)
+
+
+@MIXERS.register("gated_delta_rule")
+class GatedDeltaRule(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, dim: int, vdim: int, conv_taps: int,
+                 eps: float, names: Optional[dict] = None):
+        if num_heads <= 0 or num_kv_heads <= 0 or num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} heads do not split over {num_kv_heads} query/key heads")
+        if not 0 < dim <= ops.LINEAR_SCAN_MAX_DIM or vdim <= 0 or conv_taps < 1:
+            raise ValueError(f"gated delta rule: heads of {dim}/{vdim} (keys of up to {ops.LINEAR_SCAN_MAX_DIM}), "
+                             f"{conv_taps} taps")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.dim, self.vdim, self.taps, self.eps = int(dim), int(vdim), int(conv_taps), float(eps)
+        n = dict(q="q", k="k", v="v", q_conv="q.conv", k_conv="k.conv", v_conv="v.conv", beta="b", decay_log="A_log",
+                 decay_in="a1", decay_out="a2", decay_bias="dt_bias", gate_in="g1", gate_out="g2", norm="norm", o="o")
+        n.update(names or {})
+        self.names = n
+        self.channels = 2 * self.num_kv_heads * self.dim + self.num_heads * self.vdim   # what passes the convolution
+        self.qkv = self.decay_in = self.gate_in = self.beta = self.in_proj = None
+        self.conv = self.decay_log = self.decay_out = self.decay_bias = self.gate_out = self.norm = self.o_proj = None
+        self.conv_f = self.coef_f = self.decay_out_f = self.decay_bias_f = self.gate_out_f = self.norm_f = None
+        self.decay_rank = self.gate_rank = 0
+
+    def weight_specs(self):
+        n, C, H, G = self.names, self.hidden_size, self.num_heads, self.num_kv_heads
+        kd, vd = G * self.dim, H * self.vdim
+        r = free_size(MADE_UP_RANK)
+        return [
+            WeightSpec("qkv", (WeightSource(n["q"], (kd, C)), WeightSource(n["k"], (kd, C)), WeightSource(n["v"], (vd, C)))),
+            WeightSpec("conv", (WeightSource(n["q_conv"], (kd, self.taps)), WeightSource(n["k_conv"], (kd, self.taps)),
+                                WeightSource(n["v_conv"], (vd, self.taps)))),
+            WeightSpec("decay_in", (WeightSource(n["decay_in"], (r, C)),)),
+            WeightSpec("gate_in", (WeightSource(n["gate_in"], (r, C)),)),
+            WeightSpec("beta", (WeightSource(n["beta"], (H, C)),)),
+            WeightSpec("decay_out", (WeightSource(n["decay_out"], (H * self.dim, r)),)),
+            WeightSpec("decay_bias", (WeightSource(n["decay_bias"], (H * self.dim,)),)),
+            WeightSpec("decay_log", (WeightSource(n["decay_log"], (H,)),)),
+            WeightSpec("gate_out", (WeightSource(n["gate_out"], (vd, r)),)),
+            WeightSpec("norm", (WeightSource(n["norm"], (self.vdim,)),), init="ones"),
+            WeightSpec("o_proj", (WeightSource(n["o"], (C, vd)),)),
+        ]
+
+    def materialize(self, device, dtype):
+        self.decay_rank, self.gate_rank = self.decay_in.shape[0], self.gate_in.shape[0]
+        if self.decay_out.shape[1] != self.decay_rank or self.gate_out.shape[1] != self.gate_rank:
+            raise ValueError(f"gated delta rule: the low-rank pairs' inner sizes differ: {tuple(self.decay_in.shape)} / "
+                             f"{tuple(self.decay_out.shape)}, {tuple(self.gate_in.shape)} / {tuple(self.gate_out.shape)}")
+        # everything that reads the layer's input, as one matrix: q, k, v | decay | gate | beta
+        self.in_proj = torch.cat([self.qkv, self.decay_in, self.gate_in, self.beta], dim=0).contiguous()
+        self.qkv = self.decay_in = self.gate_in = self.beta = None
+        self.conv_f = self.conv.float().contiguous()
+        self.coef_f = torch.exp(self.decay_log.float()).contiguous()
+        self.decay_out_f = self.decay_out.float().contiguous()
+        self.decay_bias_f = self.decay_bias.float().contiguous()
+        self.gate_out_f = self.gate_out.float().contiguous()
+        self.norm_f = self.norm.float().contiguous()
+
+    def state_spec(self):
+        return StateSpec((self.num_heads, self.vdim, self.dim), torch.float32)
+
+    def further_states(self):
+        # the convolution's last inputs, kept as they were read (activations)
+        return {"conv": StateSpec((self.taps - 1, self.channels), None)} if self.taps > 1 else {}
+
+    def forward(self, ctx: StepContext, x, cache: LayerCache):
+        H, G, C3 = self.num_heads, self.num_kv_heads, self.channels
+        kd = G * self.dim
+        p = ops.linear(x, self.in_proj, out_dtype=ctx.dtype)
+        qkv = torch.empty((ctx.T, C3), dtype=ctx.dtype, device=p.device)
+        ops.short_conv(p[:, :C3], self.conv_f, cache.states.get("mixer.conv"), ctx.q_start, ctx.positions,
+                       ctx.state_slots, qkv, ctx.B, residual=False, silu=True)
+        at = C3
+        z = ops.lowrank_up(p[:, at:at + self.decay_rank], self.decay_out_f, self.decay_bias_f)
+        at += self.decay_rank
+        gate = ops.lowrank_up(p[:, at:at + self.gate_rank], self.gate_out_f)
+        at += self.gate_rank
+        o = _scan_out(ctx, H * self.vdim)
+        ops.linear_scan(qkv[:, :kd], qkv[:, kd:2 * kd], qkv[:, 2 * kd:], z, None, self.coef_f, 1.0, cache.state,
+                        ctx.q_start, ctx.positions, ctx.state_slots, o, ctx.B, num_heads=H, num_kv_heads=G, dim=self.dim,
+                        vdim=self.vdim, beta=p[:, at:at + H], unit=True, q_scale=self.dim ** -0.5)
+        y = ops.head_norm_gate(o, self.norm_f, gate, "sigmoid", self.eps, ctx.dtype, num_heads=H, vdim=self.vdim)
+        return ops.linear(y, self.o_proj, out_dtype=ctx.dtype)
+
+
+@MIXERS.register("gated_linear_attention")
+class GatedLinearAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, dim: int, vdim: int, tau: float, eps: float,
+                 names: Optional[dict] = None):
+        if num_heads <= 0 or not 0 < dim <= ops.LINEAR_SCAN_MAX_DIM or vdim <= 0 or not tau > 0:
+            raise ValueError(f"gated linear attention: {num_heads} heads of {dim}/{vdim} (keys of up to "
+                             f"{ops.LINEAR_SCAN_MAX_DIM}), tau {tau}")
+        self.hidden_size, self.num_heads, self.dim, self.vdim = int(hidden_size), int(num_heads), int(dim), int(vdim)
+        self.tau, self.eps = float(tau), float(eps)
+        n = dict(q="q", k="k", v="v", g="g", decay_in="a1", decay_out="a2", decay_bias="a2.b", norm="norm", o="o")
+        n.update(names or {})
+        self.names = n
+        self.qkvg = self.decay_in = self.in_proj = None
+        self.decay_out = self.decay_bias = self.norm = self.o_proj = None
+        self.coef_f = self.decay_out_f = self.decay_bias_f = self.norm_f = None
+        self.decay_rank = 0
+
+    def weight_specs(self):
+        n, C, H = self.names, self.hidden_size, self.num_heads
+        kd, vd = H * self.dim, H * self.vdim
+        r = free_size(MADE_UP_RANK)
+        return [
+            WeightSpec("qkvg", (WeightSource(n["q"], (kd, C)), WeightSource(n["k"], (kd, C)), WeightSource(n["v"], (vd, C)),
+                                WeightSource(n["g"], (vd, C)))),
+            WeightSpec("decay_in", (WeightSource(n["decay_in"], (r, C)),)),
+            WeightSpec("decay_out", (WeightSource(n["decay_out"], (kd, r)),)),
+            WeightSpec("decay_bias", (WeightSource(n["decay_bias"], (kd,)),)),
+            WeightSpec("norm", (WeightSource(n["norm"], (self.vdim,)),), init="ones"),
+            WeightSpec("o_proj", (WeightSource(n["o"], (C, vd)),)),
+        ]
+
+    def materialize(self, device, dtype):
+        self.decay_rank = self.decay_in.shape[0]
+        if self.decay_out.shape[1] != self.decay_rank:
+            raise ValueError(f"gated linear attention: the decay's low-rank pair is {tuple(self.decay_in.shape)} / "
+                             f"{tuple(self.decay_out.shape)}")
+        self.in_proj = torch.cat([self.qkvg, self.decay_in], dim=0).contiguous()
+        self.qkvg = self.decay_in = None
+        self.coef_f = torch.full((self.num_heads,), 1.0 / self.tau, dtype=torch.float32, device=self.in_proj.device)
+        self.decay_out_f = self.decay_out.float().contiguous()
+        self.decay_bias_f = self.decay_bias.float().contiguous()
+        self.norm_f = self.norm.float().contiguous()
+
+    def state_spec(self):
+        return StateSpec((self.num_heads, self.vdim, self.dim), torch.float32)
+
+    def forward(self, ctx: StepContext, x, cache: LayerCache):
+        H = self.num_heads
+        kd, vd = H * self.dim, H * self.vdim
+        p = ops.linear(x, self.in_proj, out_dtype=ctx.dtype)
+        at = 2 * kd + 2 * vd
+        # sigmoid(z)^(1/tau) = exp(-softplus(-z) / tau)
+        z = ops.lowrank_up(p[:, at:at + self.decay_rank], self.decay_out_f, self.decay_bias_f)
+        o = _scan_out(ctx, vd)
+        ops.linear_scan(p[:, :kd], p[:, kd:2 * kd], p[:, 2 * kd:2 * kd + vd], z, None, self.coef_f, -1.0, cache.state,
+                        ctx.q_start, ctx.positions, ctx.state_slots, o, ctx.B, num_heads=H, num_kv_heads=H, dim=self.dim,
+                        vdim=self.vdim, unit=False, q_scale=self.dim ** -0.5)
+        y = ops.head_norm_gate(o, self.norm_f, p[:, 2 * kd + vd:at], "silu", self.eps, ctx.dtype, num_heads=H,
+                               vdim=self.vdim)
+        return ops.linear(y, self.o_proj, out_dtype=ctx.dtype)

@@ -53,6 +53,31 @@ class DenseFeedForward(FeedForward):
         return ops.linear(up, self.down_proj, out_dtype=ctx.dtype)
 
 
+@FEED_FORWARDS.register("gated_dense")
+class GatedDense(FeedForward):
+    """down(act(gate(x)) * up(x)), no biases; ``activation``: "silu" or "gelu_tanh" (the tanh form of
+    gelu).  Gate and up are one matrix whose first rows are the gate."""
+
+    def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu", names: Optional[dict] = None):
+        if activation not in ops.GLU_ACTIVATIONS:
+            raise ValueError(f"unknown gate activation {activation!r}; known: {sorted(ops.GLU_ACTIVATIONS)}")
+        self.hidden_size, self.intermediate_size, self.activation = int(hidden_size), int(intermediate_size), activation
+        n = dict(gate="gate", up="up", down="down")
+        n.update(names or {})
+        self.names = n
+        self.gate_up_proj: Optional[torch.Tensor] = None
+        self.down_proj: Optional[torch.Tensor] = None
+
+    def weight_specs(self):
+        n, shape = self.names, (self.intermediate_size, self.hidden_size)
+        return [WeightSpec("gate_up_proj", (WeightSource(n["gate"], shape), WeightSource(n["up"], shape))),
+                WeightSpec("down_proj", (WeightSource(n["down"], (self.hidden_size, self.intermediate_size)),))]
+
+    def forward(self, ctx: StepContext, x):
+        act = ops.glu_act(ops.linear(x, self.gate_up_proj, out_dtype=ctx.dtype), self.activation)
+        return ops.linear(act, self.down_proj, out_dtype=ctx.dtype)
+
+
 @FEED_FORWARDS.register("swiglu")
 class SwiGLU(FeedForward):
     def __init__(self, hidden_size: int, intermediate_size: int):

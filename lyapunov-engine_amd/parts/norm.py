@@ -71,3 +71,40 @@ class RMSNorm(Norm):
         n = h.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.size), dtype=ctx.dtype, device=h.device)
         return ops.rmsnorm(h, self.weight, self.eps, out, delta=delta, rows=rows)
+
+
+@NORMS.register("group_rmsnorm")
+class GroupRMSNorm(Norm):
+    """RMS norm in groups: a row is cut into ``groups`` equal consecutive parts, each divided by its
+    own sqrt(mean(part^2) + eps), and the whole row multiplied by the weight.  All in 32-bit.  The
+    norm adds what is still to be added to the stream on its way: a tensor, float partial sums, or
+    an ``ops.ScaledBranch`` (a branch times a learned vector), in the same kernel."""
+
+    takes_scaled = True
+
+    def __init__(self, size: int, eps: float, groups: int = 1, tensor: str = "weight"):
+        if groups < 1 or size % groups:
+            raise ValueError(f"rows of {size} values do not split into {groups} equal groups")
+        self.size, self.eps, self.groups, self.tensor = int(size), float(eps), int(groups), tensor
+        self.weight: Optional[torch.Tensor] = None
+        self._weight_f: Optional[torch.Tensor] = None
+
+    def weight_specs(self):
+        return [WeightSpec("weight", (WeightSource(self.tensor, (self.size,)),), init="ones")]
+
+    @property
+    def weight_f(self) -> torch.Tensor:
+        if self._weight_f is None:
+            self._weight_f = self.weight.float().contiguous()
+        return self._weight_f
+
+    def forward(self, ctx: StepContext, h, delta=None, rows=None, out_dtype=None):
+        """``out_dtype``: the normed rows' type (None: the step's activations)."""
+        scale = None
+        if isinstance(delta, ops.ScaledBranch):
+            delta, scale = delta.y, delta.scale
+        if isinstance(delta, ops.PendingLinear):
+            delta = delta.run()
+        n = h.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, self.size), dtype=out_dtype or ctx.dtype, device=h.device)
+        return ops.group_rmsnorm(h, self.weight_f, self.groups, self.eps, out, delta=delta, scale=scale, rows=rows)

@@ -99,3 +99,63 @@ class RoutedExperts(FeedForward):
         if addend is not None:
             addend = ops.as_delta(addend, ctx.dtype)
         return ops.moe_combine(y, plan, wgt, T, addend=addend, shared=shared)
+
+
+@FEED_FORWARDS.register("group_routed_experts")
+class GroupRoutedExperts(FeedForward):
+    """Experts chosen by sigmoid scores within the best groups:
+
+        s = sigmoid(W_r x)                                 in 32-bit
+        choice scores c = s + correction; the experts form ``groups`` equal groups of neighbours, a
+        group's score is the sum of its two largest c, and only experts of the ``keep`` best groups
+        can be chosen; the ``top`` largest c among those are
+        weights: the chosen experts' s over their sum (+ 1e-20), times ``scale``
+        expert e:  y_e = W_down,e relu(W_up,e x)^2         no gate, no biases
+        out = sum over the chosen e of weight_e * y_e
+
+    The (token, choice) pairs are sorted by expert on the device; both products walk the sorted
+    tiles (``ops.moe_gemm``: the first gathers its rows by token and squares the positive part of
+    its result), the last kernel adds a token's weighted outputs in 32-bit."""
+
+    choices_log: Optional[list] = None   # as RoutedExperts.choices_log
+
+    def __init__(self, hidden_size: int, num_experts: int, top: int, intermediate_size: int, groups: int = 1,
+                 keep: int = 1, scale: float = 1.0, names: Optional[dict] = None):
+        if not 1 <= top <= num_experts or intermediate_size <= 0:
+            raise ValueError(f"routed experts: {top} of {num_experts} experts of {intermediate_size}")
+        if groups < 1 or num_experts % groups or not 1 <= keep <= groups or keep * (num_experts // groups) < top:
+            raise ValueError(f"routed experts: {num_experts} experts in {groups} groups of which {keep} are kept "
+                             f"cannot give {top} choices")
+        self.hidden_size, self.num_experts, self.top = int(hidden_size), int(num_experts), int(top)
+        self.intermediate_size, self.groups, self.keep, self.scale = int(intermediate_size), int(groups), int(keep), float(scale)
+        n = dict(router="router", correction="correction", expert="e{j}.", up="up", down="down")
+        n.update(names or {})
+        self.names = n
+        self.router = self.correction = self.up = self.down = None
+        self.router_f = self.correction_f = None
+
+    def weight_specs(self):
+        n, E, I, H = self.names, self.num_experts, self.intermediate_size, self.hidden_size
+        ups = tuple(WeightSource(n["expert"].format(j=j) + n["up"], (I, H)) for j in range(E))
+        downs = tuple(WeightSource(n["expert"].format(j=j) + n["down"], (H, I)) for j in range(E))
+        return [WeightSpec("router", (WeightSource(n["router"], (E, H)),)),
+                WeightSpec("correction", (WeightSource(n["correction"], (E,)),)),
+                WeightSpec("up", ups), WeightSpec("down", downs)]
+
+    def materialize(self, device, dtype):
+        E, I, H = self.num_experts, self.intermediate_size, self.hidden_size
+        self.router_f = self.router.float().contiguous()
+        self.correction_f = self.correction.float().contiguous()
+        self.router = None
+        self.up = self.up.view(E, I, H)
+        self.down = self.down.view(E, H, I)
+
+    def forward(self, ctx: StepContext, x):
+        """-> float [1, T, hidden] (one slice of partial sums)."""
+        idx, wgt = ops.moe_route_grouped(x, self.router_f, self.correction_f, self.top, self.groups, self.keep, self.scale)
+        if GroupRoutedExperts.choices_log is not None:
+            GroupRoutedExperts.choices_log.append(idx)
+        plan = ops.moe_sort(idx, self.num_experts)
+        act = ops.moe_gemm(x, self.up, plan, gated=False, gather=True, relu2=True)
+        y = ops.moe_gemm(act, self.down, plan, gated=False)
+        return ops.moe_combine(y, plan, wgt, x.shape[0])

@@ -21,6 +21,7 @@ import torch
 
 from ..config.registry import load_config
 from ..models.decoder import DecoderModel, build_model
+from ..parts.base import shape_fits
 from ..utils import log
 from .safetensors_io import open_model_files
 
@@ -70,7 +71,7 @@ def check_tensors(model: DecoderModel, present: dict) -> None:
     missing = sorted(n for n in expected if n not in present)
     unexpected = sorted(n for n in present if n not in expected and not model.ignorable(n))
     wrong = sorted((n, tuple(present[n]), expected[n][0]) for n in expected
-                   if n in present and tuple(present[n]) != tuple(expected[n][0]))
+                   if n in present and not shape_fits(tuple(present[n]), tuple(expected[n][0])))
     if not (missing or unexpected or wrong):
         return
     lines = ["the model's tensors do not match its configuration:"]
@@ -80,7 +81,8 @@ def check_tensors(model: DecoderModel, present: dict) -> None:
         lines.append(f"  unexpected ({len(unexpected)}): " + ", ".join(unexpected))
     if wrong:
         lines.append(f"  wrong shape ({len(wrong)}): " +
-                     ", ".join(f"{n} is {list(got)}, expected {list(want)}" for n, got, want in wrong))
+                     ", ".join(f"{n} is {list(got)}, expected {[w if w >= 0 else 'any' for w in want]}"
+                               for n, got, want in wrong))
     raise WeightError("\n".join(lines))
 
 

@@ -18,6 +18,7 @@ import torch
 
 from ..config.registry import ARCHITECTURES, architecture_of
 from ..models.decoder import build_model
+from ..parts.base import made_up_shape
 from .safetensors_io import write_safetensors
 
 _STORE = {"bfloat16": torch.bfloat16, "float32": torch.float32, "float16": torch.float16}
@@ -39,7 +40,7 @@ def random_tensors(model, seed: int, dtype: torch.dtype, init_std: Optional[floa
     for name, (shape, init) in model.expected_tensors().items():
         gen = torch.Generator(device=device)
         gen.manual_seed(_tensor_seed(seed, name))
-        t = torch.randn(shape, generator=gen, dtype=torch.float32, device=device)
+        t = torch.randn(made_up_shape(shape), generator=gen, dtype=torch.float32, device=device)
         if init == "ones":
             t = 1.0 + t * nstd
         elif init == "normal":
