@@ -191,41 +191,65 @@ def gated_dense(h, w, pre):
     return (gelu_tanh(h @ w[pre + "gate"].T) * (h @ w[pre + "up"].T)) @ w[pre + "down"].T
 
 
-def choose_experts(s, correction, r):
+def choose_experts(s, correction, r, margin_out=None):
     """s [T, E] sigmoid scores -> (chosen [T, top] indices, weights [T, top]).  Experts are chosen by
     s + correction among the ``keep`` groups (of ``count`` groups of neighbours) whose two largest
-    choice scores add up highest; the weights are the chosen experts' plain s over their sum, times r.scale."""
+    choice scores add up highest; the weights are the chosen experts' plain s over their sum, times r.scale.
+    ``margin_out``: a list that receives, per token, how clear the choice was (the smaller of the gap
+    between the last kept and the first dropped group and the gap between the last chosen and the
+    first not chosen expert)."""
     T, E = s.shape
     c = s + correction
     count, keep = r["groups"]["count"], r["groups"]["keep"]
     per = E // count
     grouped = c.reshape(T, count, per)
     gscore = torch.topk(grouped, min(2, per), -1).values.sum(-1)
+    gsorted = torch.sort(gscore, -1, descending=True).values
     kept = torch.topk(gscore, keep, -1).indices
     allowed = torch.zeros(T, count, dtype=torch.bool)
     allowed.scatter_(1, kept, True)
     c = c.masked_fill(~allowed[:, :, None].expand(T, count, per).reshape(T, E), float("-inf"))
+    csorted = torch.sort(c, -1, descending=True).values
     chosen = torch.topk(c, r["top"], -1).indices
+    if margin_out is not None:
+        big = torch.full((T,), float("inf"), dtype=s.dtype)
+        g_gap = gsorted[:, keep - 1] - gsorted[:, keep] if keep < count else big
+        e_gap = csorted[:, r["top"] - 1] - csorted[:, r["top"]] if r["top"] < keep * per else big
+        margin_out.append(torch.minimum(g_gap, e_gap))
+    return chosen, route_weights(s, chosen, r)
+
+
+def route_weights(s, chosen, r):
     ws = torch.gather(s, 1, chosen)
-    return chosen, ws / (ws.sum(-1, keepdim=True) + 1e-20) * r["scale"]
+    return ws / (ws.sum(-1, keepdim=True) + 1e-20) * r["scale"]
 
 
-def expert_mixture(h, w, pre, mlp):
+def expert_mixture(h, w, pre, mlp, chosen=None, note=None):
+    """``chosen`` [T, top]: experts to use instead of the router's own choice (the weights still come
+    from the scores); ``note``: a dict that receives the own choice and its margins."""
     r = mlp["router"]
     s = torch.sigmoid(h @ w[pre + "router"].T)
-    chosen, weights = choose_experts(s, w[pre + "correction"], r)
+    margins = []
+    own, weights = choose_experts(s, w[pre + "correction"], r, margins)
+    if note is not None:
+        note.update(chosen=own, margin=margins[0])
+    if chosen is not None:
+        own, weights = chosen.long(), route_weights(s, chosen.long(), r)
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
-        for j, e in enumerate(chosen[t].tolist()):
+        for j, e in enumerate(own[t].tolist()):
             a = torch.relu(h[t] @ w[f"{pre}e{e}.up"].T) ** 2
             out[t] += weights[t, j] * (a @ w[f"{pre}e{e}.down"].T)
     return out
 
 
 # ------------------------------------------------------------------ the model
-def forward(tokens, w, cfg, layers_out=None):
+def forward(tokens, w, cfg, layers_out=None, chosen=None, notes=None):
     """float64 logits [T, vocab] of one whole sequence; ``layers_out``: a list that receives the
-    residual stream after every layer."""
+    residual stream after every layer; ``chosen``: one tensor [T, top] per layer with a mixture of
+    experts, in order, to be used instead of the routers' own choices; ``notes``: a list that
+    receives a dict (own choice, margins) per such layer."""
+    moe_at = 0
     T, C = len(tokens), cfg["width"]
     eps, groups = cfg["norm"]["eps"], cfg["norm"]["groups"]
     positions = list(range(T))
@@ -247,7 +271,11 @@ def forward(tokens, w, cfg, layers_out=None):
             if layer["mlp"]["kind"] == "dense":
                 y = gated_dense(h, w, p + "mlp.")
             else:
-                y = expert_mixture(h, w, p + "mlp.", layer["mlp"])
+                note = {} if notes is not None else None
+                y = expert_mixture(h, w, p + "mlp.", layer["mlp"], None if chosen is None else chosen[moe_at], note)
+                moe_at += 1
+                if notes is not None:
+                    notes.append(note)
             x = x + y * w[p + "ls2"]
         if layers_out is not None:
             layers_out.append(x.clone())
