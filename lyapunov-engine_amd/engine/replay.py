@@ -19,12 +19,13 @@ MAX_LIVE_REQUESTS = 4
 
 class TraceReplayer:
     def __init__(self, model_dir: str, dtype: str, max_tokens: int, block_size: int = 16, device: str = "cuda:0",
-                 cache_groups=None, max_model_len: Optional[int] = None):
-        """``max_model_len``: the longest a request may become; by default what the pool holds (a model
+                 cache_groups=None, max_model_len: Optional[int] = None, num_state_slots: int = MAX_LIVE_REQUESTS):
+        """``num_state_slots``: how many requests may be live at once (a model with state per request
+        keeps that many slots).  ``max_model_len``: the longest a request may become; by default what the pool holds (a model
         whose layers all give pages back behind a window could run further on the same pool)."""
         num_blocks = max(1, -(-max_tokens // block_size))
         self.core = EngineCore.from_folder(model_dir, dtype=dtype, device=device, num_blocks=num_blocks,
-                                           block_size=block_size, num_state_slots=MAX_LIVE_REQUESTS,
+                                           block_size=block_size, num_state_slots=num_state_slots,
                                            cache_groups=cache_groups,
                                            max_model_len=max_model_len or num_blocks * block_size)
         self._ids: dict = {}
