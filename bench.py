@@ -115,6 +115,30 @@ DESIGN_SIZES = {
 }
 
 
+# Tonilix models with layers of a real model's sizes: gated-delta layers with a gelu-gated dense
+# feed-forward in turn with layers of attention beside gated linear attention and a mixture of
+# relu-squared experts whose chosen experts together have the dense feed-forward's weights.  Beside
+# each stands the Faledra model of equal width, depth and feed-forward weights: the closest design
+# (recurrent and attention layers in turn, a filter over time in every layer, state slots beside pages).
+def tonilix_shape(width, heads, kv_heads, dim, layers, vocab, ff, experts, top):
+    rec = max(1, width // 128)
+
+    def delta():
+        return dict(type="channel_delta", mlp=dict(kind="dense", ff=ff),
+                    mixer=dict(heads=rec, kv_heads=max(1, rec // 2), dim=128, vdim=128, conv=4))
+
+    def pair():
+        return dict(type="parallel",
+                    mlp=dict(kind="moe", expert=dict(ff=ff * 3 // (2 * top)),
+                             router=dict(experts=experts, top=top, scale=2.5, groups=dict(count=8, keep=4))),
+                    mixer=dict(left=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5,
+                                         q_temp=dict(coef=0.1, every=1024)),
+                               right=dict(heads=max(1, rec // 2), dim=64, vdim=128, tau=16.0), left_scale=1.0, right_scale=1.0))
+
+    return dict(architecture="Tonilix", vocab=vocab, width=width, norm=dict(eps=1e-5, groups=8),
+                layers=[pair() if i % 2 else delta() for i in range(layers)])
+
+
 def build_engine_from_config(raw, dtype, num_blocks, max_num_seqs, block_size, budget, max_model_len):
     """An engine for any registered architecture's config.json contents, with random weights."""
     import torch
@@ -142,6 +166,15 @@ def build_engine_from_config(raw, dtype, num_blocks, max_num_seqs, block_size, b
     return engine, cfg
 
 
+TONILIX_SIZES = {
+    "small": (tonilix_shape(1024, 16, 4, 64, 8, 32000, 4096, 16, 4), DESIGN_SIZES["small"][0]),
+    "1b": (tonilix_shape(2048, 32, 8, 64, 16, 128256, 8192, 32, 4), DESIGN_SIZES["1b"][0]),
+    "wide": (tonilix_shape(4096, 32, 8, 128, 8, 128256, 14336, 32, 4), DESIGN_SIZES["wide"][0]),
+}
+# what stands beside a design's sizes
+BESIDE = {"faledra": "llama", "ronupel": "llama", "tonilix": "faledra"}
+
+
 class _Vocab:
     """What the measuring functions read of a configuration."""
 
@@ -150,16 +183,18 @@ class _Vocab:
 
 
 def run_design(args):
-    """Prefill and decode speed of another design's sizes, each beside the Llama shape of equal size."""
+    """Prefill and decode speed of another design's sizes, each beside a model of equal size: the Llama
+    shape, or for Tonilix the Faledra model."""
     import torch
 
     context, block_size, out = 2304, 16, {}
     design = args.design
-    sizes = {"faledra": DESIGN_SIZES, "ronupel": RONUPEL_SIZES}[design]
+    sizes = {"faledra": DESIGN_SIZES, "ronupel": RONUPEL_SIZES, "tonilix": TONILIX_SIZES}[design]
+    beside = BESIDE[design]
     for size in (args.size.split(",") if args.size else sorted(sizes)):
-        other, llama = sizes[size]
+        other, second = sizes[size]
         out[size] = {}
-        for name, raw in ((design, other), ("llama", llama)):
+        for name, raw in ((design, other), (beside, second)):
             engine, _ = build_engine_from_config(raw, args.dtype, 8 * (context // block_size + 1) + 64 + 2048 // block_size,
                                                  8, block_size, budget=8192, max_model_len=context)
             cfg = _Vocab(engine)
@@ -178,7 +213,7 @@ def run_design(args):
             torch.cuda.empty_cache()
     first = out[sorted(out)[0]]
     print(json.dumps({
-        "metric": f"{design.capitalize()} beside the Llama shape of equal size: prefill and decode tok/s", "unit": "tok/s",
+        "metric": f"{design.capitalize()} beside the {beside.capitalize()} model of equal size: prefill and decode tok/s", "unit": "tok/s",
         "value": first[design]["decode_b8_ctx2048_tok_s"], "n_gpus": 1, "steps": min(args.steps, 64),
         "warmup": min(args.warmup, 8), "ms_per_step": first[design]["decode_b8_ms"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
@@ -398,9 +433,9 @@ def main():
                     help="mixed: the continuous batch of BASELINE.json configs[3] instead of the headline")
     ap.add_argument("--skip-points", action="store_true", help="only the headline decode and the prefill")
     ap.add_argument("--skip-check", action="store_true", help="no comparison of bfloat16 logits with a 32-bit run")
-    ap.add_argument("--design", default="llama", choices=["llama", "faledra", "ronupel"],
-                    help="faledra, ronupel: that design's prefill and decode speed at a few sizes, each beside the "
-                         "Llama shape of equal size, instead of the headline")
+    ap.add_argument("--design", default="llama", choices=["llama", "faledra", "ronupel", "tonilix"],
+                    help="faledra, ronupel, tonilix: that design's prefill and decode speed at a few sizes, each beside "
+                         "the Llama shape (Tonilix: the Faledra model) of equal size, instead of the headline")
     ap.add_argument("--size", default="", help="with another --design: which sizes, with commas (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
