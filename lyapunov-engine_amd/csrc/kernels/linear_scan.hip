@@ -14,9 +14,9 @@
 //   * linear_scan: the state is kept transposed, [slot][head][vdim][dim], and lives in registers:
 //     a column of S (one value of vdim) belongs to L neighbouring lanes that hold DPL key channels
 //     each; the two dot products of a token are sums inside a lane and over those L lanes.  The
-//     step's tokens of a request are walked in order; what does not depend on the state (unit
-//     vectors, decays, sigmoid of beta) is worked out for kScanChunk tokens at a time, side by side,
-//     into LDS.  A workgroup takes (a block of columns, a head, a request); columns do not depend
+//     step's tokens of a request are walked in order; what does not depend on the state (decays,
+//     the lengths of queries and keys, sigmoid of beta) is worked out for a chunk of tokens at a time,
+//     side by side by all threads, into LDS.  A workgroup takes (a block of columns, a head, a request); columns do not depend
 //     on each other.  The slot is read unless the request stands at position 0, and written back.
 //   * head_norm_gate: every head's o over vdim divided by its root mean square, times a weight
 //     shared by the heads, times sigmoid or silu of a gate's pre-activation.
@@ -28,7 +28,11 @@
 
 namespace lyp {
 
-constexpr int kScanChunk = 8;
+// Tokens staged at a time: what a token needs besides the state (decays, keys, queries, values, beta)
+// is worked out for this many tokens side by side, by all threads, so that memory's latency is paid
+// once a chunk and not once a token.
+__host__ __device__ inline int scan_chunk(int Dp) { return Dp <= 128 ? 32 : 16; }
+constexpr int kScanPad = 4;   // floats between the staged rows, so that neighbouring tokens start in other banks
 
 __device__ __forceinline__ float scan_softplus(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 __device__ __forceinline__ float scan_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
@@ -41,17 +45,22 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, float* __restrict__ out, int ldo, int H,
     int G, int D, int V, int L, int unit, float q_scale) {
   extern __shared__ __attribute__((aligned(16))) float s_scan[];
-  const int Dp = L * DPL;                      // key channels with the padding
-  const int cpb = blockDim.x / L;              // columns a workgroup
-  float* sk = s_scan;                          // [chunk][Dp]
-  float* sq = sk + kScanChunk * Dp;
-  float* sg = sq + kScanChunk * Dp;
-  float* sv = sg + kScanChunk * Dp;            // [chunk][cpb]
-  float* sb = sv + kScanChunk * cpb;           // [chunk]
+  const int Dp = L * DPL;                      // key channels with the padding: a power of two
+  const int ld = Dp + kScanPad;
+  const int chunk = scan_chunk(Dp);
+  const int cpb = blockDim.x / L;              // columns a workgroup: a power of two
+  const int dp_shift = __ffs(Dp) - 1, cpb_shift = __ffs(cpb) - 1;
+  float* sk = s_scan;                          // [chunk][ld]   keys as they come
+  float* sq = sk + chunk * ld;                 //               queries as they come
+  float* sg = sq + chunk * ld;                 //               decays
+  float* sv = sg + chunk * ld;                 // [chunk][cpb]  this workgroup's columns of the values
+  float* sb = sv + chunk * cpb;                // [chunk]       sigmoid(beta)
+  float* sfq = sb + chunk;                     // [chunk]       what a query is multiplied by (unit length, the constant)
+  float* sfk = sfq + chunk;                    // [chunk]       what a key is multiplied by
   const int b = blockIdx.z, h = blockIdx.y;
   const int q0 = q_start[b], n = q_start[b + 1] - q0;
   if (n <= 0) return;
-  const int tid = threadIdx.x, lane = tid % kWave, wave = tid / kWave, waves = blockDim.x / kWave;
+  const int tid = threadIdx.x;
   const int l = tid % L, cl = tid / L;
   const int col = blockIdx.x * cpb + cl;
   const int d0 = l * DPL;
@@ -63,47 +72,61 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
   for (int i = 0; i < DPL; ++i) S[i] = (!fresh && col < V && d0 + i < D) ? st[d0 + i] : 0.f;
   const float a_h = coef[h];
 
-  for (int c0 = 0; c0 < n; c0 += kScanChunk) {
-    const int cn = min(kScanChunk, n - c0);
-    // a wave a token: unit vectors and decays over the key channels
-    for (int j = wave; j < cn; j += waves) {
+  for (int c0 = 0; c0 < n; c0 += chunk) {
+    const int cn = min(chunk, n - c0);
+    for (int idx = tid; idx < (cn << dp_shift); idx += blockDim.x) {
+      const int j = idx >> dp_shift, d = idx & (Dp - 1);
       const size_t row = static_cast<size_t>(q0 + c0 + j);
-      float ssq = 0.f, ssk = 0.f;
-      for (int d = lane; d < Dp; d += kWave) {
-        float qq = 0.f, kk = 0.f, gg = 1.f;
-        if (d < D) {
-          qq = to_f32(q[row * ldq + kvh * D + d]);
-          kk = to_f32(k[row * ldk + kvh * D + d]);
-          const float zz = z[row * ldz + h * D + d] + (zbias != nullptr ? zbias[h * D + d] : 0.f);
-          gg = expf(-a_h * scan_softplus(sign * zz));
-        }
-        ssq += qq * qq;
-        ssk += kk * kk;
-        sq[j * Dp + d] = qq;
-        sk[j * Dp + d] = kk;
-        sg[j * Dp + d] = gg;
+      float qq = 0.f, kk = 0.f, gg = 1.f;
+      if (d < D) {
+        qq = to_f32(q[row * ldq + kvh * D + d]);
+        kk = to_f32(k[row * ldk + kvh * D + d]);
+        const float zz = z[row * ldz + h * D + d] + (zbias != nullptr ? zbias[h * D + d] : 0.f);
+        gg = expf(-a_h * scan_softplus(sign * zz));
       }
-      float fq = q_scale, fk = 1.f;
-      if (unit) {
-        fq = q_scale / sqrtf(wave_sum(ssq) + 1e-6f);
-        fk = 1.0f / sqrtf(wave_sum(ssk) + 1e-6f);
-      }
-      for (int d = lane; d < Dp; d += kWave) {   // a lane rescales what it wrote itself
-        sq[j * Dp + d] *= fq;
-        sk[j * Dp + d] *= fk;
-      }
+      sq[j * ld + d] = qq;
+      sk[j * ld + d] = kk;
+      sg[j * ld + d] = gg;
     }
-    for (int idx = tid; idx < cn * cpb; idx += blockDim.x) {
-      const int j = idx / cpb, c = blockIdx.x * cpb + idx % cpb;
+    for (int idx = tid; idx < (cn << cpb_shift); idx += blockDim.x) {
+      const int j = idx >> cpb_shift, c = blockIdx.x * cpb + (idx & (cpb - 1));
       sv[idx] = c < V ? to_f32(v[static_cast<size_t>(q0 + c0 + j) * ldv + h * V + c]) : 0.f;
     }
-    if (DELTA && tid < cn) sb[tid] = scan_sigmoid(to_f32(beta[static_cast<size_t>(q0 + c0 + tid) * ldb + h]));
+    if (tid < cn) {
+      if (DELTA) sb[tid] = scan_sigmoid(to_f32(beta[static_cast<size_t>(q0 + c0 + tid) * ldb + h]));
+      if (!unit) {
+        sfq[tid] = q_scale;
+        sfk[tid] = 1.f;
+      }
+    }
+    if (unit) {
+      __syncthreads();
+      // four neighbouring lanes a token: the squares of its query and key, a quarter each
+      for (int j = tid / 4; j < cn; j += blockDim.x / 4) {
+        float ssq = 0.f, ssk = 0.f;
+        for (int f = tid % 4; f < Dp / 4; f += 4) {
+          const f32x4 q4 = *reinterpret_cast<const f32x4*>(sq + j * ld + 4 * f);
+          const f32x4 k4 = *reinterpret_cast<const f32x4*>(sk + j * ld + 4 * f);
+          ssq += q4[0] * q4[0] + q4[1] * q4[1] + q4[2] * q4[2] + q4[3] * q4[3];
+          ssk += k4[0] * k4[0] + k4[1] * k4[1] + k4[2] * k4[2] + k4[3] * k4[3];
+        }
+        ssq += __shfl_xor(ssq, 1, kWave);
+        ssk += __shfl_xor(ssk, 1, kWave);
+        ssq += __shfl_xor(ssq, 2, kWave);
+        ssk += __shfl_xor(ssk, 2, kWave);
+        if (tid % 4 == 0) {
+          sfq[j] = q_scale / sqrtf(ssq + 1e-6f);
+          sfk[j] = 1.0f / sqrtf(ssk + 1e-6f);
+        }
+      }
+    }
     __syncthreads();
     for (int j = 0; j < cn; ++j) {
-      const float* kj = sk + j * Dp + d0;
-      const float* qj = sq + j * Dp + d0;
-      const float* gj = sg + j * Dp + d0;
-      float u = sv[j * cpb + cl];
+      const float* kj = sk + j * ld + d0;
+      const float* qj = sq + j * ld + d0;
+      const float* gj = sg + j * ld + d0;
+      const float fk = sfk[j], fq = sfq[j];
+      float u = sv[(j << cpb_shift) + cl];
       float r0 = 0.f, r1 = 0.f;
 #pragma unroll
       for (int i = 0; i < DPL; i += 4) {
@@ -119,8 +142,9 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
       if constexpr (DELTA) {
         float r = r0 + r1;
         for (int off = 1; off < L; off <<= 1) r += __shfl_xor(r, off, kWave);
-        u = sb[j] * (u - r);
+        u = sb[j] * (u - fk * r);
       }
+      u *= fk;
       float o0 = 0.f, o1 = 0.f;
 #pragma unroll
       for (int i = 0; i < DPL; i += 4) {
@@ -133,7 +157,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
       }
       float o = o0 + o1;
       for (int off = 1; off < L; off <<= 1) o += __shfl_xor(o, off, kWave);
-      if (l == 0 && col < V) out[static_cast<size_t>(q0 + c0 + j) * ldo + h * V + col] = o;
+      if (l == 0 && col < V) out[static_cast<size_t>(q0 + c0 + j) * ldo + h * V + col] = o * fq;
     }
     __syncthreads();   // the chunk's staging is read to the end before the next overwrites it
   }
@@ -208,12 +232,12 @@ int lyp_linear_scan_lanes(int D) {
 }
 
 // q, k [rows, >= G*D] and v [rows, >= H*V] of dtype, rows ldq / ldk / ldv apart; z float [rows, >= H*D] (ldz apart);
-// zbias float [H*D] or null; coef float [H]; beta [rows, >= H] of dtype (ldb apart; the delta rule only: delta != 0);
+// zbias float [H*D] or null; coef float [H]; rows: all requests' rows together; beta [rows, >= H] of dtype (ldb apart; the delta rule only: delta != 0);
 // state float [slots, H, V, D]; out float [rows, >= H*V] (ldo apart).  Request b owns rows q_start[b] .. q_start[b+1].
 int lyp_linear_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, int dtype, const float* z,
                     int ldz, const float* zbias, const float* coef, float sign, const void* beta, int ldb,
                     float* state, const int32_t* q_start, const int32_t* positions, const int32_t* slots, float* out,
-                    int ldo, int B, int H, int G, int D, int V, int delta, int unit, float q_scale,
+                    int ldo, int rows, int B, int H, int G, int D, int V, int delta, int unit, float q_scale,
                     hipStream_t stream) {
   LYP_REQUIRE(B > 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && V > 0, "linear_scan: B=%d H=%d G=%d D=%d V=%d", B, H, G,
               D, V);
@@ -226,13 +250,15 @@ int lyp_linear_scan(const void* q, int ldq, const void* k, int ldk, const void* 
   const int dpl = D <= 64 ? 16 : 32;
   // columns a workgroup: as few as fill a wave when there are few (request, head) pairs, so that
   // the launch has workgroups for the machine; up to four waves otherwise
+  // (a request of many rows keeps its waves together all the same: they share the chunk's staging)
   int threads = 256;
-  while (threads > 64 && static_cast<long long>(B) * H * ((V * L + threads - 1) / threads) < 2LL * compute_units())
+  while (threads > 64 && rows < 16LL * B &&
+         static_cast<long long>(B) * H * ((V * L + threads - 1) / threads) < 2LL * compute_units())
     threads /= 2;
   while (threads > 64 && threads / 2 >= V * L) threads /= 2;
   const int cpb = threads / L;
   dim3 grid((V + cpb - 1) / cpb, H, B);
-  const size_t lds = static_cast<size_t>(kScanChunk) * (3 * L * dpl + cpb + 1) * sizeof(float);
+  const size_t lds = static_cast<size_t>(scan_chunk(L * dpl)) * (3 * (L * dpl + kScanPad) + cpb + 3) * sizeof(float);
 #define LYP_SCAN(T, DPLV, DEL)                                                                                      \
   linear_scan_kernel<T, DPLV, DEL><<<grid, threads, lds, stream>>>(                                                 \
       static_cast<const T*>(q), ldq, static_cast<const T*>(k), ldk, static_cast<const T*>(v), ldv, z, ldz, zbias,   \

@@ -346,42 +346,93 @@ __global__ __launch_bounds__(kSortThreads) void moe_sort_kernel(
 // two largest choice scores (its one score when a group is one expert), and only experts of the
 // `keep` best groups can be chosen.  The `top` largest choice scores among those are taken (of
 // equal ones the first); their weights are s over the sum of the chosen s (+ 1e-20), times scale.
-// One wave per row: the lanes share the inner dimension of every expert's product in a fixed
-// order, lane 0 then chooses.
-constexpr int kGroupedRows = 4;   // rows (waves) a workgroup
+// A wave forms a row's product with a block of experts at a time (the block's loads all in flight,
+// the lanes sharing the inner dimension in a fixed order that does not depend on the launch); a
+// workgroup's four waves take four rows, or, when the step has few rows, share one row's experts.
+// Then one wave per row chooses: group scores a lane each, maxima over the wave.
+constexpr int kGroupedRows = 4;   // waves a workgroup
+constexpr int kRouteBlock = 8;    // experts whose products a wave forms side by side
+
+template <typename T>
+__device__ __forceinline__ f32x4 route_load4(const T* p);
+template <>
+__device__ __forceinline__ f32x4 route_load4<float>(const float* p) {
+  return *reinterpret_cast<const f32x4*>(p);
+}
+template <>
+__device__ __forceinline__ f32x4 route_load4<bf16_t>(const bf16_t* p) {
+  const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+  return f32x4{static_cast<float>(v[0]), static_cast<float>(v[1]), static_cast<float>(v[2]), static_cast<float>(v[3])};
+}
+
+__device__ __forceinline__ ArgMax wave_argmax(ArgMax m) {
+#pragma unroll
+  for (int off = kWave / 2; off > 0; off >>= 1) {
+    ArgMax o;
+    o.v = __shfl_xor(m.v, off, kWave);
+    o.i = __shfl_xor(m.i, off, kWave);
+    m = better(m, o);
+  }
+  return m;
+}
 
 template <typename T>
 __global__ __launch_bounds__(kGroupedRows* kWave) void moe_route_grouped_kernel(
     const T* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ correction, int rows, int E,
-    int K, int top, int n_groups, int keep, float scale, int32_t* __restrict__ idx, float* __restrict__ wgt) {
+    int K, int top, int n_groups, int keep, float scale, int32_t* __restrict__ idx, float* __restrict__ wgt, int rpb,
+    int vec_ok) {
   __shared__ float s_score[kGroupedRows][kMostExperts];    // s
-  __shared__ float s_choice[kGroupedRows][kMostExperts];   // s + correction
-  __shared__ int s_open[kGroupedRows][kMostExperts];       // 1: may still be chosen
+  __shared__ float s_choice[kGroupedRows][kMostExperts];   // s + correction; minus infinity once chosen
   const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
-  const int row = blockIdx.x * kGroupedRows + wave;
-  if (row >= rows) return;
-  const T* xr = x + static_cast<size_t>(row) * ldx;
-  for (int e = 0; e < E; ++e) {
-    const float* we = w + static_cast<size_t>(e) * K;
-    float acc = 0.f;
-    for (int k = lane; k < K; k += kWave) acc += to_f32(xr[k]) * we[k];
-    acc = wave_sum(acc);
-    if (lane == 0) {
-      const float s = 1.0f / (1.0f + expf(-acc));
-      s_score[wave][e] = s;
-      s_choice[wave][e] = s + (correction != nullptr ? correction[e] : 0.f);
-      s_open[wave][e] = 0;
+  const int slot = wave % rpb, share = wave / rpb, shares = kGroupedRows / rpb;
+  const int row = blockIdx.x * rpb + slot;
+  if (row < rows) {
+    const T* xr = x + static_cast<size_t>(row) * ldx;
+    for (int e0 = share * kRouteBlock; e0 < E; e0 += shares * kRouteBlock) {
+      float acc[kRouteBlock];
+      const float* we[kRouteBlock];
+#pragma unroll
+      for (int j = 0; j < kRouteBlock; ++j) {
+        acc[j] = 0.f;
+        we[j] = w + static_cast<size_t>(min(e0 + j, E - 1)) * K;   // past the last expert: worked out, not kept
+      }
+      if (vec_ok) {
+        for (int k = lane * 4; k < K; k += kWave * 4) {
+          const f32x4 xv = route_load4<T>(xr + k);
+#pragma unroll
+          for (int j = 0; j < kRouteBlock; ++j) {
+            const f32x4 wv = *reinterpret_cast<const f32x4*>(we[j] + k);
+            acc[j] += xv[0] * wv[0] + xv[1] * wv[1] + xv[2] * wv[2] + xv[3] * wv[3];
+          }
+        }
+      } else {
+        for (int k = lane; k < K; k += kWave) {
+          const float xv = to_f32(xr[k]);
+#pragma unroll
+          for (int j = 0; j < kRouteBlock; ++j) acc[j] += xv * we[j][k];
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < kRouteBlock; ++j) {
+        const float sum = wave_sum(acc[j]);
+        if (lane == 0 && e0 + j < E) {
+          const float sg = 1.0f / (1.0f + expf(-sum));
+          s_score[slot][e0 + j] = sg;
+          s_choice[slot][e0 + j] = sg + (correction != nullptr ? correction[e0 + j] : 0.f);
+        }
+      }
     }
   }
-  if (lane != 0) return;
-  const float* c = s_choice[wave];
-  int* open = s_open[wave];
+  __syncthreads();
+  if (share != 0 || row >= rows) return;
+  float* c = s_choice[slot];
   const int per = E / n_groups;
-  float gscore[64];   // there are at most 64 groups
-  for (int g = 0; g < n_groups; ++g) {
-    float a = LYP_NEG_INF, b = LYP_NEG_INF;   // the two largest
+  // a lane a group: the sum of its two largest choice scores (its one score for a group of one)
+  float gs = LYP_NEG_INF;
+  if (lane < n_groups) {
+    float a = LYP_NEG_INF, b = LYP_NEG_INF;
     for (int i = 0; i < per; ++i) {
-      const float v = c[g * per + i];
+      const float v = c[lane * per + i];
       if (v > a) {
         b = a;
         a = v;
@@ -389,27 +440,33 @@ __global__ __launch_bounds__(kGroupedRows* kWave) void moe_route_grouped_kernel(
         b = v;
       }
     }
-    gscore[g] = per > 1 ? a + b : a;
+    gs = per > 1 ? a + b : a;
   }
-  unsigned long long taken = 0ull;
+  unsigned long long kept = 0ull;
+  bool mine_taken = lane >= n_groups;
   for (int n = 0; n < keep; ++n) {
-    int best = -1;
-    for (int g = 0; g < n_groups; ++g)
-      if (!((taken >> g) & 1ull) && (best < 0 || gscore[g] > gscore[best])) best = g;
-    taken |= 1ull << best;
-    for (int i = 0; i < per; ++i) open[best * per + i] = 1;
+    ArgMax m{mine_taken ? LYP_NEG_INF : gs, mine_taken ? 0x7fffffff : lane};
+    m = wave_argmax(m);
+    kept |= 1ull << m.i;
+    if (lane == m.i) mine_taken = true;
   }
   float total = 0.f;
+  int chosen = 0;   // lane n keeps the n-th choice
   for (int n = 0; n < top; ++n) {
-    int best = -1;
-    for (int e = 0; e < E; ++e)
-      if (open[e] && (best < 0 || c[e] > c[best])) best = e;
-    open[best] = 0;
-    idx[static_cast<size_t>(row) * top + n] = best;
-    total += s_score[wave][best];
+    ArgMax m{LYP_NEG_INF, 0x7fffffff};
+    for (int e = lane; e < E; e += kWave)
+      if ((kept >> (e / per)) & 1ull) m = better(m, ArgMax{c[e], e});
+    m = wave_argmax(m);
+    if (lane == n) chosen = m.i;
+    if (lane == 0) c[m.i] = LYP_NEG_INF;
+    total += s_score[slot][m.i];
+    // the wave's lanes run together: the store above is seen by the next round's reads
+    __builtin_amdgcn_wave_barrier();
   }
-  for (int n = 0; n < top; ++n)
-    wgt[static_cast<size_t>(row) * top + n] = s_score[wave][idx[static_cast<size_t>(row) * top + n]] / (total + 1e-20f) * scale;
+  if (lane < top) {
+    idx[static_cast<size_t>(row) * top + lane] = chosen;
+    wgt[static_cast<size_t>(row) * top + lane] = s_score[slot][chosen] / (total + 1e-20f) * scale;
+  }
 }
 
 
@@ -810,19 +867,25 @@ int lyp_moe_route(const float* z, const float* bias, int rows, int E, int top, i
 int lyp_moe_route_grouped(const void* x, int ldx, int dtype, const float* w, const float* correction, int rows, int E,
                           int K, int top, int n_groups, int keep, float scale, int32_t* idx, float* wgt,
                           hipStream_t stream) {
-  LYP_REQUIRE(rows >= 0 && E > 0 && E <= kMostExperts && K > 0 && ldx >= K && top > 0,
-              "moe_route_grouped: %d rows, %d experts (at most %d), inner size %d, %d chosen", rows, E, kMostExperts, K, top);
+  LYP_REQUIRE(rows >= 0 && E > 0 && E <= kMostExperts && K > 0 && ldx >= K && top > 0 && top <= kMostTop,
+              "moe_route_grouped: %d rows, %d experts (at most %d), inner size %d, %d chosen (at most %d)", rows, E,
+              kMostExperts, K, top, kMostTop);
   LYP_REQUIRE(n_groups >= 1 && n_groups <= 64 && E % n_groups == 0 && keep >= 1 && keep <= n_groups &&
                   keep * (E / n_groups) >= top,
               "moe_route_grouped: %d experts in %d groups of which %d are kept cannot give %d choices", E, n_groups, keep, top);
   if (rows == 0) return 0;
-  const int blocks = (rows + kGroupedRows - 1) / kGroupedRows;
+  // few rows: a workgroup's waves share one row's experts, so that the router matrix is pulled through by many
+  const int rpb = rows >= 2 * compute_units() ? kGroupedRows : 1;
+  const int blocks = (rows + rpb - 1) / rpb;
+  const size_t esz = dtype == kF32 ? 4 : 2;
+  const int vec_ok = K % 4 == 0 && ldx % 4 == 0 && reinterpret_cast<uintptr_t>(x) % (4 * esz) == 0 &&
+                     reinterpret_cast<uintptr_t>(w) % 16 == 0;
   if (dtype == kF32)
     moe_route_grouped_kernel<float><<<blocks, kGroupedRows * kWave, 0, stream>>>(
-        static_cast<const float*>(x), ldx, w, correction, rows, E, K, top, n_groups, keep, scale, idx, wgt);
+        static_cast<const float*>(x), ldx, w, correction, rows, E, K, top, n_groups, keep, scale, idx, wgt, rpb, vec_ok);
   else if (dtype == kBF16)
     moe_route_grouped_kernel<bf16_t><<<blocks, kGroupedRows * kWave, 0, stream>>>(
-        static_cast<const bf16_t*>(x), ldx, w, correction, rows, E, K, top, n_groups, keep, scale, idx, wgt);
+        static_cast<const bf16_t*>(x), ldx, w, correction, rows, E, K, top, n_groups, keep, scale, idx, wgt, rpb, vec_ok);
   else
     LYP_REQUIRE(false, "moe_route_grouped: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("moe_route_grouped");

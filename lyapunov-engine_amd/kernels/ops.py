@@ -143,7 +143,7 @@ def core() -> ctypes.CDLL:
         lib.lyp_linear_scan_lanes.argtypes = [c_int]
         lib.lyp_linear_scan.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int,
                                         c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
-                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                         c_float, c_void_p]
         lib.lyp_head_norm_gate.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
                                            c_int, c_float, c_int, c_void_p]
@@ -1692,7 +1692,7 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tens
     _check(lib.lyp_linear_scan(_p(q), q.stride(0), _p(k), k.stride(0), _p(v), v.stride(0), _code(q.dtype), _p(z),
                                z.stride(0), _p(zbias), _p(coef), float(sign), _p(beta),
                                beta.stride(0) if beta is not None else 0, _p(state), _p(q_start), _p(positions), _p(slots),
-                               _p(out), out.stride(0), B, H, G, dim, vdim, int(beta is not None), int(unit),
+                               _p(out), out.stride(0), T, B, H, G, dim, vdim, int(beta is not None), int(unit),
                                float(q_scale), _stream()), lib)
     return out
 
