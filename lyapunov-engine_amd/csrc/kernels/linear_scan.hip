@@ -6,14 +6,15 @@
 //                             S <- S + k_t u^T                                 o_t = S^T q_t
 //
 // with a decay per head and key channel, g = exp(-coef_head * softplus(sign * (z + bias))), which
-// covers exp(-A softplus(z + b)) (sign +1, coef A) and sigmoid(z + b)^(1/tau) (sign -1, coef 1/tau).
+// covers exp(-A softplus(z + b)) (sign +1, coef A) and sigmoid(z + b)^(1/tau) (sign -1, coef 1/tau);
+// sign 0 says that z holds the decays themselves (lowrank_up works them out on its way).
 // Queries and keys may be made unit vectors per head first (x / sqrt(sum x^2 + 1e-6)); queries
 // take a constant factor.  Decays, unit vectors, gates, sums and the state are 32-bit; q, k, v come
 // in the activations' type.
 //
 //   * linear_scan: the state is kept transposed, [slot][head][vdim][dim], and lives in registers:
-//     a column of S (one value of vdim) belongs to L neighbouring lanes that hold DPL key channels
-//     each; the two dot products of a token are sums inside a lane and over those L lanes.  The
+//     a column of S (one value of vdim) belongs to L neighbouring lanes (up to 16) that hold DPL key
+//     channels each; the two dot products of a token are sums inside a lane and over those L lanes.  The
 //     step's tokens of a request are walked in order; what does not depend on the state (decays,
 //     the lengths of queries and keys, sigmoid of beta) is worked out for a chunk of tokens at a time,
 //     side by side by all threads, into LDS.  A workgroup takes (a block of columns, a head, a request); columns do not depend
@@ -31,23 +32,44 @@ namespace lyp {
 // Tokens staged at a time: what a token needs besides the state (decays, keys, queries, values, beta)
 // is worked out for this many tokens side by side, by all threads, so that memory's latency is paid
 // once a chunk and not once a token.
-__host__ __device__ inline int scan_chunk(int Dp) { return Dp <= 128 ? 32 : 16; }
+__host__ __device__ inline int scan_chunk(int Dp) { return Dp <= 128 ? 32 : (Dp <= 256 ? 16 : 8); }
 constexpr int kScanPad = 4;   // floats between the staged rows, so that neighbouring tokens start in other banks
 
 __device__ __forceinline__ float scan_softplus(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 __device__ __forceinline__ float scan_sigmoid(float v) { return 1.0f / (1.0f + expf(-v)); }
 
-template <typename T, int DPL, bool DELTA>
+// The sum over a group of L neighbouring lanes (L a power of two up to 16, groups aligned), by
+// lane permutations inside a row of 16; every lane of the group gets it.
+template <int CTRL>
+__device__ __forceinline__ float scan_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float group_sum(float v, int L) {
+  if (L > 1) v += scan_dpp<0xB1>(v);    // neighbours: lanes 1 0 3 2 of every four
+  if (L > 2) v += scan_dpp<0x4E>(v);    // lanes 2 3 0 1 of every four
+  if (L > 4) v += scan_dpp<0x141>(v);   // every eight mirrored
+  if (L > 8) v += scan_dpp<0x140>(v);   // every sixteen mirrored
+  return v;
+}
+
+// With S' = diag(g) S the token's two products with the state are both taken from S' in one pass,
+//   r = k . S',  p = q . S';   u = beta (v - r)  (u = v without the delta rule);
+//   S = S' + k u^T;  o = q . S = p + (q . k) u,
+// and q . k does not depend on the state: it is staged with the lengths.
+// STAGE: keys, queries and decays a thread fetches in one round (and half as many values): 16 for steps
+// of long portions, 4 for steps of single tokens and short portions, which then need few registers
+// and many workgroups fit a compute unit.
+template <typename T, int DPL, bool DELTA, int STAGE>
 __global__ __launch_bounds__(256) void linear_scan_kernel(
     const T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
     const float* __restrict__ z, int ldz, const float* __restrict__ zbias, const float* __restrict__ coef, float sign,
     const T* __restrict__ beta, int ldb, float* __restrict__ state, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, float* __restrict__ out, int ldo, int H,
-    int G, int D, int V, int L, int unit, float q_scale) {
+    int G, int D, int V, int L, int unit, float q_scale, int chunk) {
   extern __shared__ __attribute__((aligned(16))) float s_scan[];
   const int Dp = L * DPL;                      // key channels with the padding: a power of two
   const int ld = Dp + kScanPad;
-  const int chunk = scan_chunk(Dp);
+  const int l_shift = __ffs(L) - 1;
   const int cpb = blockDim.x / L;              // columns a workgroup: a power of two
   const int dp_shift = __ffs(Dp) - 1, cpb_shift = __ffs(cpb) - 1;
   float* sk = s_scan;                          // [chunk][ld]   keys as they come
@@ -57,6 +79,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
   float* sb = sv + chunk * cpb;                // [chunk]       sigmoid(beta)
   float* sfq = sb + chunk;                     // [chunk]       what a query is multiplied by (unit length, the constant)
   float* sfk = sfq + chunk;                    // [chunk]       what a key is multiplied by
+  float* sqk = sfk + chunk;                    // [chunk]       query . key, as they come
   const int b = blockIdx.z, h = blockIdx.y;
   const int q0 = q_start[b], n = q_start[b + 1] - q0;
   if (n <= 0) return;
@@ -72,92 +95,162 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
   for (int i = 0; i < DPL; ++i) S[i] = (!fresh && col < V && d0 + i < D) ? st[d0 + i] : 0.f;
   const float a_h = coef[h];
 
+  constexpr int kStage = STAGE, kStageV = STAGE / 2;
+  // What a chunk's tokens bring is fetched into registers kStage values a thread at a time, all loads
+  // in flight together, and staged in LDS from there.  A workgroup whose threads cover a whole chunk
+  // in one such round fetches the next chunk before it walks the current one's tokens, so that
+  // memory's latency passes meanwhile.
+  T rq[kStage], rk[kStage];
+  float rz[kStage];
+  T rv[kStageV];
+  T rb = from_f32<T>(0.f);
+  const int per_round = kStage * blockDim.x;
+  const bool ahead = (chunk << dp_shift) <= per_round && (chunk << cpb_shift) <= kStageV * static_cast<int>(blockDim.x);
+  auto fetch = [&](int c0, int cn, int base) {
+#pragma unroll
+    for (int u = 0; u < kStage; ++u) {
+      const int idx = base + u * blockDim.x + tid;
+      const int j = idx >> dp_shift, d = idx & (Dp - 1);
+      rq[u] = rk[u] = from_f32<T>(0.f);
+      rz[u] = 0.f;
+      if (j < cn && d < D) {
+        const size_t row = static_cast<size_t>(q0 + c0 + j);
+        rq[u] = q[row * ldq + kvh * D + d];
+        rk[u] = k[row * ldk + kvh * D + d];
+        rz[u] = z[row * ldz + h * D + d];
+      }
+    }
+  };
+  auto fetch_values = [&](int c0, int cn) {
+#pragma unroll
+    for (int u = 0; u < kStageV; ++u) {
+      const int idx = u * blockDim.x + tid;
+      const int j = idx >> cpb_shift, c = blockIdx.x * cpb + (idx & (cpb - 1));
+      rv[u] = (j < cn && c < V) ? v[static_cast<size_t>(q0 + c0 + j) * ldv + h * V + c] : from_f32<T>(0.f);
+    }
+    if (DELTA && tid < cn) rb = beta[static_cast<size_t>(q0 + c0 + tid) * ldb + h];
+  };
+  auto stash = [&](int cn, int base) {
+#pragma unroll
+    for (int u = 0; u < kStage; ++u) {
+      const int idx = base + u * blockDim.x + tid;
+      const int j = idx >> dp_shift, d = idx & (Dp - 1);
+      if (j < cn) {
+        float gg = 1.f;
+        if (d < D) gg = sign == 0.f ? rz[u] : expf(-a_h * scan_softplus(sign * (rz[u] + (zbias != nullptr ? zbias[h * D + d] : 0.f))));
+        // a lane's channels four by four in planes, so that a plane's read takes neighbouring lanes to neighbouring words
+        const int at = j * ld + ((((d & (DPL - 1)) >> 2) << (l_shift + 2)) | ((d / DPL) << 2) | (d & 3));
+        sq[at] = to_f32(rq[u]);
+        sk[at] = to_f32(rk[u]);
+        sg[at] = gg;
+      }
+    }
+  };
+  auto stash_values = [&](int cn) {
+#pragma unroll
+    for (int u = 0; u < kStageV; ++u) {
+      const int idx = u * blockDim.x + tid;
+      if (idx < (cn << cpb_shift)) sv[idx] = to_f32(rv[u]);
+    }
+    if (DELTA && tid < cn) sb[tid] = scan_sigmoid(to_f32(rb));
+  };
+  if (ahead) {
+    fetch(0, min(chunk, n), 0);
+    fetch_values(0, min(chunk, n));
+  }
+
   for (int c0 = 0; c0 < n; c0 += chunk) {
     const int cn = min(chunk, n - c0);
-    for (int idx = tid; idx < (cn << dp_shift); idx += blockDim.x) {
-      const int j = idx >> dp_shift, d = idx & (Dp - 1);
-      const size_t row = static_cast<size_t>(q0 + c0 + j);
-      float qq = 0.f, kk = 0.f, gg = 1.f;
-      if (d < D) {
-        qq = to_f32(q[row * ldq + kvh * D + d]);
-        kk = to_f32(k[row * ldk + kvh * D + d]);
-        const float zz = z[row * ldz + h * D + d] + (zbias != nullptr ? zbias[h * D + d] : 0.f);
-        gg = expf(-a_h * scan_softplus(sign * zz));
+    if (ahead) {
+      stash(cn, 0);
+      stash_values(cn);
+    } else {
+      for (int base = 0; base < (cn << dp_shift); base += per_round) {
+        fetch(c0, cn, base);
+        stash(cn, base);
       }
-      sq[j * ld + d] = qq;
-      sk[j * ld + d] = kk;
-      sg[j * ld + d] = gg;
-    }
-    for (int idx = tid; idx < (cn << cpb_shift); idx += blockDim.x) {
-      const int j = idx >> cpb_shift, c = blockIdx.x * cpb + (idx & (cpb - 1));
-      sv[idx] = c < V ? to_f32(v[static_cast<size_t>(q0 + c0 + j) * ldv + h * V + c]) : 0.f;
-    }
-    if (tid < cn) {
-      if (DELTA) sb[tid] = scan_sigmoid(to_f32(beta[static_cast<size_t>(q0 + c0 + tid) * ldb + h]));
-      if (!unit) {
-        sfq[tid] = q_scale;
-        sfk[tid] = 1.f;
+      for (int idx = tid; idx < (cn << cpb_shift); idx += blockDim.x) {
+        const int j = idx >> cpb_shift, c = blockIdx.x * cpb + (idx & (cpb - 1));
+        sv[idx] = c < V ? to_f32(v[static_cast<size_t>(q0 + c0 + j) * ldv + h * V + c]) : 0.f;
       }
+      if (DELTA && tid < cn) sb[tid] = scan_sigmoid(to_f32(beta[static_cast<size_t>(q0 + c0 + tid) * ldb + h]));
     }
-    if (unit) {
-      __syncthreads();
-      // four neighbouring lanes a token: the squares of its query and key, a quarter each
-      for (int j = tid / 4; j < cn; j += blockDim.x / 4) {
-        float ssq = 0.f, ssk = 0.f;
-        for (int f = tid % 4; f < Dp / 4; f += 4) {
-          const f32x4 q4 = *reinterpret_cast<const f32x4*>(sq + j * ld + 4 * f);
-          const f32x4 k4 = *reinterpret_cast<const f32x4*>(sk + j * ld + 4 * f);
-          ssq += q4[0] * q4[0] + q4[1] * q4[1] + q4[2] * q4[2] + q4[3] * q4[3];
-          ssk += k4[0] * k4[0] + k4[1] * k4[1] + k4[2] * k4[2] + k4[3] * k4[3];
-        }
-        ssq += __shfl_xor(ssq, 1, kWave);
-        ssk += __shfl_xor(ssk, 1, kWave);
-        ssq += __shfl_xor(ssq, 2, kWave);
-        ssk += __shfl_xor(ssk, 2, kWave);
-        if (tid % 4 == 0) {
-          sfq[j] = q_scale / sqrtf(ssq + 1e-6f);
-          sfk[j] = 1.0f / sqrtf(ssk + 1e-6f);
-        }
+    __syncthreads();
+    // four neighbouring lanes a token: the squares of its query and key and their product, a quarter each
+    for (int j = tid / 4; j < cn; j += blockDim.x / 4) {
+      float ssq = 0.f, ssk = 0.f, sqkv = 0.f;
+      for (int f = tid % 4; f < Dp / 4; f += 4) {
+        const f32x4 q4 = *reinterpret_cast<const f32x4*>(sq + j * ld + 4 * f);
+        const f32x4 k4 = *reinterpret_cast<const f32x4*>(sk + j * ld + 4 * f);
+        ssq += q4[0] * q4[0] + q4[1] * q4[1] + q4[2] * q4[2] + q4[3] * q4[3];
+        ssk += k4[0] * k4[0] + k4[1] * k4[1] + k4[2] * k4[2] + k4[3] * k4[3];
+        sqkv += q4[0] * k4[0] + q4[1] * k4[1] + q4[2] * k4[2] + q4[3] * k4[3];
+      }
+      ssq = group_sum(ssq, 4);
+      ssk = group_sum(ssk, 4);
+      sqkv = group_sum(sqkv, 4);
+      if (tid % 4 == 0) {
+        sfq[j] = unit ? q_scale / sqrtf(ssq + 1e-6f) : q_scale;
+        sfk[j] = unit ? 1.0f / sqrtf(ssk + 1e-6f) : 1.f;
+        sqk[j] = sqkv;
       }
     }
     __syncthreads();
-    for (int j = 0; j < cn; ++j) {
-      const float* kj = sk + j * ld + d0;
-      const float* qj = sq + j * ld + d0;
-      const float* gj = sg + j * ld + d0;
-      const float fk = sfk[j], fq = sfq[j];
-      float u = sv[(j << cpb_shift) + cl];
-      float r0 = 0.f, r1 = 0.f;
+    if (ahead && c0 + chunk < n) {
+      fetch(c0 + chunk, min(chunk, n - c0 - chunk), 0);
+      fetch_values(c0 + chunk, min(chunk, n - c0 - chunk));
+    }
+    // a token's operands are read from LDS while the token before it is worked on
+    f32x4 g4[DPL / 4], q4[DPL / 4], k4[DPL / 4], ng[DPL / 4], nq[DPL / 4], nk[DPL / 4];
+    float fk, fq, qk, u, bt = 1.f, nfk, nfq, nqk, nu, nbt = 1.f;
+    auto read = [&](int j, f32x4 (&g_)[DPL / 4], f32x4 (&q_)[DPL / 4], f32x4 (&k_)[DPL / 4], float& fk_, float& fq_, float& qk_,
+                    float& u_, float& bt_) {
+      const int at = j * ld + 4 * l;
 #pragma unroll
-      for (int i = 0; i < DPL; i += 4) {
-        const f32x4 g4 = *reinterpret_cast<const f32x4*>(gj + i);
+      for (int i = 0; i < DPL / 4; ++i) {
+        g_[i] = *reinterpret_cast<const f32x4*>(sg + at + ((i << l_shift) << 2));
+        q_[i] = *reinterpret_cast<const f32x4*>(sq + at + ((i << l_shift) << 2));
+        k_[i] = *reinterpret_cast<const f32x4*>(sk + at + ((i << l_shift) << 2));
+      }
+      fk_ = sfk[j];
+      fq_ = sfq[j];
+      qk_ = sqk[j];
+      u_ = sv[(j << cpb_shift) + cl];
+      if constexpr (DELTA) bt_ = sb[j];
+    };
+    auto work = [&](int j, const f32x4 (&g_)[DPL / 4], const f32x4 (&q_)[DPL / 4], const f32x4 (&k_)[DPL / 4], float fk_,
+                    float fq_, float qk_, float u_, float bt_) {
+      float r0 = 0.f, r1 = 0.f, p0 = 0.f, p1 = 0.f;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) S[i + e] *= g4[e];
+      for (int i = 0; i < DPL / 4; ++i) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) S[4 * i + e] *= g_[i][e];
         if constexpr (DELTA) {
-          const f32x4 k4 = *reinterpret_cast<const f32x4*>(kj + i);
-          r0 += S[i] * k4[0] + S[i + 2] * k4[2];
-          r1 += S[i + 1] * k4[1] + S[i + 3] * k4[3];
+          r0 += S[4 * i] * k_[i][0] + S[4 * i + 2] * k_[i][2];
+          r1 += S[4 * i + 1] * k_[i][1] + S[4 * i + 3] * k_[i][3];
         }
+        p0 += S[4 * i] * q_[i][0] + S[4 * i + 2] * q_[i][2];
+        p1 += S[4 * i + 1] * q_[i][1] + S[4 * i + 3] * q_[i][3];
       }
-      if constexpr (DELTA) {
-        float r = r0 + r1;
-        for (int off = 1; off < L; off <<= 1) r += __shfl_xor(r, off, kWave);
-        u = sb[j] * (u - fk * r);
-      }
-      u *= fk;
-      float o0 = 0.f, o1 = 0.f;
+      const float p = group_sum(p0 + p1, L);
+      if constexpr (DELTA) u_ = bt_ * (u_ - fk_ * group_sum(r0 + r1, L));
+      u_ *= fk_;
 #pragma unroll
-      for (int i = 0; i < DPL; i += 4) {
-        const f32x4 k4 = *reinterpret_cast<const f32x4*>(kj + i);
-        const f32x4 q4 = *reinterpret_cast<const f32x4*>(qj + i);
+      for (int i = 0; i < DPL / 4; ++i) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) S[i + e] += k4[e] * u;
-        o0 += S[i] * q4[0] + S[i + 2] * q4[2];
-        o1 += S[i + 1] * q4[1] + S[i + 3] * q4[3];
+        for (int e = 0; e < 4; ++e) S[4 * i + e] += k_[i][e] * u_;
       }
-      float o = o0 + o1;
-      for (int off = 1; off < L; off <<= 1) o += __shfl_xor(o, off, kWave);
-      if (l == 0 && col < V) out[static_cast<size_t>(q0 + c0 + j) * ldo + h * V + col] = o * fq;
+      if (l == 0 && col < V) out[static_cast<size_t>(q0 + c0 + j) * ldo + h * V + col] = fq_ * (p + qk_ * u_);
+    };
+    // two tokens a round, their operands in two sets of registers in turn
+    read(0, g4, q4, k4, fk, fq, qk, u, bt);
+    for (int j = 0; j < cn; j += 2) {
+      read(min(j + 1, cn - 1), ng, nq, nk, nfk, nfq, nqk, nu, nbt);
+      work(j, g4, q4, k4, fk, fq, qk, u, bt);
+      if (j + 1 < cn) {
+        read(min(j + 2, cn - 1), g4, q4, k4, fk, fq, qk, u, bt);
+        work(j + 1, ng, nq, nk, nfk, nfq, nqk, nu, nbt);
+      }
     }
     __syncthreads();   // the chunk's staging is read to the end before the next overwrites it
   }
@@ -196,7 +289,8 @@ constexpr int kLowRows = 8;
 template <typename T>
 __global__ __launch_bounds__(256) void lowrank_up_kernel(const T* __restrict__ mid, int ldm, const float* __restrict__ w,
                                                          const float* __restrict__ bias, float* __restrict__ out,
-                                                         int rows, int N, int R) {
+                                                         int rows, int N, int R, const float* __restrict__ coef,
+                                                         float sign, int per_head) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   const int t0 = blockIdx.y * kLowRows;
   if (n >= N) return;
@@ -211,9 +305,11 @@ __global__ __launch_bounds__(256) void lowrank_up_kernel(const T* __restrict__ m
     for (int j = 0; j < kLowRows; ++j)
       if (t0 + j < rows) acc[j] += x * to_f32(mid[static_cast<size_t>(t0 + j) * ldm + r]);
   }
+  const float a = coef != nullptr ? coef[n / per_head] : 0.f;
 #pragma unroll
   for (int j = 0; j < kLowRows; ++j)
-    if (t0 + j < rows) out[static_cast<size_t>(t0 + j) * N + n] = acc[j];
+    if (t0 + j < rows)
+      out[static_cast<size_t>(t0 + j) * N + n] = coef != nullptr ? expf(-a * scan_softplus(sign * acc[j])) : acc[j];
 }
 
 }  // namespace lyp
@@ -222,10 +318,17 @@ using namespace lyp;
 
 extern "C" {
 
+// Key channels a lane holds of its column of the state, for key heads of D values: as few as keep a
+// column within the 16 lanes whose sums go by lane permutations (0: D is too large).
+static int scan_channels_per_lane(int D) {
+  if (D <= 0 || D > 512) return 0;
+  return D <= 128 ? 8 : (D <= 256 ? 16 : 32);
+}
+
 // Lanes a column of the state is spread over, for key heads of D values (0: D is too large).
 int lyp_linear_scan_lanes(int D) {
-  if (D <= 0 || D > 256) return 0;
-  const int dpl = D <= 64 ? 16 : 32;
+  const int dpl = scan_channels_per_lane(D);
+  if (dpl == 0) return 0;
   int L = 1;
   while (L * dpl < D) L *= 2;
   return L;
@@ -242,12 +345,12 @@ int lyp_linear_scan(const void* q, int ldq, const void* k, int ldk, const void* 
   LYP_REQUIRE(B > 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && V > 0, "linear_scan: B=%d H=%d G=%d D=%d V=%d", B, H, G,
               D, V);
   const int L = lyp_linear_scan_lanes(D);
-  LYP_REQUIRE(L > 0, "linear_scan: key heads of up to 256 values, not %d", D);
+  LYP_REQUIRE(L > 0 && L <= 16, "linear_scan: key heads of up to 512 values, not %d", D);
   LYP_REQUIRE(ldq >= G * D && ldk >= G * D && ldv >= H * V && ldz >= H * D && ldo >= H * V && (!delta || ldb >= H),
               "linear_scan: rows too short for %d/%d heads of %d/%d", H, G, D, V);
   LYP_REQUIRE(!delta || beta != nullptr, "linear_scan: the delta rule needs beta");
   LYP_REQUIRE(H <= 65535 && B <= 65535, "linear_scan: too many heads or requests for one launch");
-  const int dpl = D <= 64 ? 16 : 32;
+  const int dpl = scan_channels_per_lane(D);
   // columns a workgroup: as few as fill a wave when there are few (request, head) pairs, so that
   // the launch has workgroups for the machine; up to four waves otherwise
   // (a request of many rows keeps its waves together all the same: they share the chunk's staging)
@@ -258,15 +361,26 @@ int lyp_linear_scan(const void* q, int ldq, const void* k, int ldk, const void* 
   while (threads > 64 && threads / 2 >= V * L) threads /= 2;
   const int cpb = threads / L;
   dim3 grid((V + cpb - 1) / cpb, H, B);
-  const size_t lds = static_cast<size_t>(scan_chunk(L * dpl)) * (3 * (L * dpl + kScanPad) + cpb + 3) * sizeof(float);
-#define LYP_SCAN(T, DPLV, DEL)                                                                                      \
-  linear_scan_kernel<T, DPLV, DEL><<<grid, threads, lds, stream>>>(                                                 \
+  // few rows a request (single tokens, short portions): a short chunk, so that many workgroups fit a compute unit
+  const bool brief = rows < 16LL * B;
+  const int chunk = brief ? (rows <= B ? 2 : std::min(8, scan_chunk(L * dpl))) : scan_chunk(L * dpl);
+  const size_t lds = static_cast<size_t>(chunk) * (3 * (L * dpl + kScanPad) + cpb + 4) * sizeof(float);
+#define LYP_SCAN_S(T, DPLV, DEL, ST)                                                                                \
+  linear_scan_kernel<T, DPLV, DEL, ST><<<grid, threads, lds, stream>>>(                                               \
       static_cast<const T*>(q), ldq, static_cast<const T*>(k), ldk, static_cast<const T*>(v), ldv, z, ldz, zbias,   \
       coef, sign, static_cast<const T*>(beta), ldb, state, q_start, positions, slots, out, ldo, H, G, D, V, L, unit, \
-      q_scale)
+      q_scale, chunk)
+#define LYP_SCAN(T, DPLV, DEL)              \
+  do {                                      \
+    if (brief) LYP_SCAN_S(T, DPLV, DEL, 4); \
+    else LYP_SCAN_S(T, DPLV, DEL, 16);      \
+  } while (0)
 #define LYP_SCAN_T(T)                          \
   do {                                         \
-    if (dpl == 16) {                           \
+    if (dpl == 8) {                            \
+      if (delta) LYP_SCAN(T, 8, true);         \
+      else LYP_SCAN(T, 8, false);              \
+    } else if (dpl == 16) {                    \
       if (delta) LYP_SCAN(T, 16, true);        \
       else LYP_SCAN(T, 16, false);             \
     } else {                                   \
@@ -279,6 +393,7 @@ int lyp_linear_scan(const void* q, int ldq, const void* k, int ldk, const void* 
   else LYP_REQUIRE(false, "linear_scan: unknown dtype %d", dtype);
 #undef LYP_SCAN_T
 #undef LYP_SCAN
+#undef LYP_SCAN_S
   LYP_LAUNCH_CHECK("linear_scan");
   return 0;
 }
@@ -306,17 +421,19 @@ int lyp_head_norm_gate(const float* o, const float* w, const void* gate, int ldg
 }
 
 // mid [rows, >= R] of dtype (ldm apart); w float [N, R]; bias float [N] or null; out float [rows, N].
+// coef float [N / per_head] or null: the result y becomes the decay exp(-coef[n / per_head] * softplus(sign * y)).
 int lyp_lowrank_up(const void* mid, int ldm, int dtype, const float* w, const float* bias, float* out, int rows, int N,
-                   int R, hipStream_t stream) {
+                   int R, const float* coef, float sign, int per_head, hipStream_t stream) {
+  LYP_REQUIRE(coef == nullptr || (per_head > 0 && N % per_head == 0), "lowrank_up: %d values in heads of %d", N, per_head);
   LYP_REQUIRE(rows >= 0 && N > 0 && R > 0 && ldm >= R, "lowrank_up: rows=%d N=%d R=%d ldm=%d", rows, N, R, ldm);
   if (rows == 0) return 0;
   const int threads = N >= 256 ? 256 : 64 * ((N + 63) / 64);
   dim3 grid((N + threads - 1) / threads, (rows + kLowRows - 1) / kLowRows);
   LYP_REQUIRE(grid.y <= 65535, "lowrank_up: too many rows for one launch");
   if (dtype == kF32)
-    lowrank_up_kernel<float><<<grid, threads, 0, stream>>>(static_cast<const float*>(mid), ldm, w, bias, out, rows, N, R);
+    lowrank_up_kernel<float><<<grid, threads, 0, stream>>>(static_cast<const float*>(mid), ldm, w, bias, out, rows, N, R, coef, sign, per_head);
   else if (dtype == kBF16)
-    lowrank_up_kernel<bf16_t><<<grid, threads, 0, stream>>>(static_cast<const bf16_t*>(mid), ldm, w, bias, out, rows, N, R);
+    lowrank_up_kernel<bf16_t><<<grid, threads, 0, stream>>>(static_cast<const bf16_t*>(mid), ldm, w, bias, out, rows, N, R, coef, sign, per_head);
   else
     LYP_REQUIRE(false, "lowrank_up: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("lowrank_up");

@@ -148,7 +148,7 @@ def core() -> ctypes.CDLL:
         lib.lyp_head_norm_gate.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
                                            c_int, c_float, c_int, c_void_p]
         lib.lyp_lowrank_up.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                       c_void_p]
+                                       c_void_p, c_float, c_int, c_void_p]
         lib.lyp_moe_route_grouped.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                               c_int, c_int, c_float, c_void_p, c_void_p, c_void_p]
         _core = lib
@@ -1660,7 +1660,7 @@ def qkv_bias_temper_kv(pre: torch.Tensor, bias: torch.Tensor | None, positions: 
     return q
 
 
-LINEAR_SCAN_MAX_DIM = 256    # key channels a head of ``linear_scan`` may have
+LINEAR_SCAN_MAX_DIM = 512    # key channels a head of ``linear_scan`` may have
 
 
 def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor, zbias: torch.Tensor | None,
@@ -1669,7 +1669,7 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tens
                 vdim: int, beta: torch.Tensor | None = None, unit: bool = False, q_scale: float = 1.0) -> torch.Tensor:
     """The recurrence with a matrix state per head over the step's rows, request by request, in order:
     S <- diag(g) S (+ the delta rule's correction when ``beta`` is given) + k v^T, out = S^T q, with
-    g = exp(-coef[head] * softplus(sign * (z + zbias))).  q, k [T, G dim] and v [T, H vdim] are
+    g = exp(-coef[head] * softplus(sign * (z + zbias))); sign 0: z holds the decays themselves.  q, k [T, G dim] and v [T, H vdim] are
     activations (column ranges of wider tensors are fine), z float [T, H dim], beta [T, H] activations
     (before its sigmoid), state float [slots, H, vdim, dim] (a head's matrix transposed), out float
     [T, H vdim].  ``unit``: q and k become unit vectors per head first; q is multiplied by ``q_scale``."""
@@ -1716,18 +1716,25 @@ def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, ki
     return out
 
 
-def lowrank_up(mid: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
-    """float [T, N] = mid @ w.T (+ bias) in 32-bit: mid [T, R] activations (a column range is fine), w float [N, R]."""
+def lowrank_up(mid: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
+               decay_coef: torch.Tensor | None = None, decay_sign: float = 1.0) -> torch.Tensor:
+    """float [T, N] = mid @ w.T (+ bias) in 32-bit: mid [T, R] activations (a column range is fine), w float [N, R].
+    With ``decay_coef`` (float, one value per head of N / len values) the result y becomes the decay
+    exp(-coef[head] * softplus(decay_sign * y)) that ``linear_scan`` takes with sign 0."""
     _rows_view(mid, "lowrank_up")
-    _dev(w, bias)
-    _f32(w, bias)
+    _dev(w, bias, decay_coef)
+    _f32(w, bias, decay_coef)
     T, R = mid.shape
     N = w.shape[0]
     if w.shape[1] != R or (bias is not None and bias.numel() != N):
         raise KernelError(f"lowrank_up: mid {tuple(mid.shape)}, w {tuple(w.shape)}")
     out = torch.empty((T, N), dtype=torch.float32, device=mid.device)
     lib = core()
-    _check(lib.lyp_lowrank_up(_p(mid), mid.stride(0), _code(mid.dtype), _p(w), _p(bias), _p(out), T, N, R, _stream()), lib)
+    heads = decay_coef.numel() if decay_coef is not None else 1
+    if N % heads:
+        raise KernelError(f"lowrank_up: {N} values do not split over {heads} heads")
+    _check(lib.lyp_lowrank_up(_p(mid), mid.stride(0), _code(mid.dtype), _p(w), _p(bias), _p(out), T, N, R, _p(decay_coef),
+                              float(decay_sign), N // heads, _stream()), lib)
     return out
 
 

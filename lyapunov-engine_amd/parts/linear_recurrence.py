@@ -113,12 +113,12 @@ class GatedDeltaRule(Mixer):
         ops.short_conv(p[:, :C3], self.conv_f, cache.states.get("mixer.conv"), ctx.q_start, ctx.positions,
                        ctx.state_slots, qkv, ctx.B, residual=False, silu=True)
         at = C3
-        z = ops.lowrank_up(p[:, at:at + self.decay_rank], self.decay_out_f, self.decay_bias_f)
+        g = ops.lowrank_up(p[:, at:at + self.decay_rank], self.decay_out_f, self.decay_bias_f, decay_coef=self.coef_f)
         at += self.decay_rank
         gate = ops.lowrank_up(p[:, at:at + self.gate_rank], self.gate_out_f)
         at += self.gate_rank
         o = _scan_out(ctx, H * self.vdim)
-        ops.linear_scan(qkv[:, :kd], qkv[:, kd:2 * kd], qkv[:, 2 * kd:], z, None, self.coef_f, 1.0, cache.state,
+        ops.linear_scan(qkv[:, :kd], qkv[:, kd:2 * kd], qkv[:, 2 * kd:], g, None, self.coef_f, 0.0, cache.state,
                         ctx.q_start, ctx.positions, ctx.state_slots, o, ctx.B, num_heads=H, num_kv_heads=G, dim=self.dim,
                         vdim=self.vdim, beta=p[:, at:at + H], unit=True, q_scale=self.dim ** -0.5)
         y = ops.head_norm_gate(o, self.norm_f, gate, "sigmoid", self.eps, ctx.dtype, num_heads=H, vdim=self.vdim)
@@ -177,9 +177,10 @@ class GatedLinearAttention(Mixer):
         p = ops.linear(x, self.in_proj, out_dtype=ctx.dtype)
         at = 2 * kd + 2 * vd
         # sigmoid(z)^(1/tau) = exp(-softplus(-z) / tau)
-        z = ops.lowrank_up(p[:, at:at + self.decay_rank], self.decay_out_f, self.decay_bias_f)
+        g = ops.lowrank_up(p[:, at:at + self.decay_rank], self.decay_out_f, self.decay_bias_f, decay_coef=self.coef_f,
+                           decay_sign=-1.0)
         o = _scan_out(ctx, vd)
-        ops.linear_scan(p[:, :kd], p[:, kd:2 * kd], p[:, 2 * kd:2 * kd + vd], z, None, self.coef_f, -1.0, cache.state,
+        ops.linear_scan(p[:, :kd], p[:, kd:2 * kd], p[:, 2 * kd:2 * kd + vd], g, None, self.coef_f, 0.0, cache.state,
                         ctx.q_start, ctx.positions, ctx.state_slots, o, ctx.B, num_heads=H, num_kv_heads=H, dim=self.dim,
                         vdim=self.vdim, unit=False, q_scale=self.dim ** -0.5)
         y = ops.head_norm_gate(o, self.norm_f, p[:, 2 * kd + vd:at], "silu", self.eps, ctx.dtype, num_heads=H,

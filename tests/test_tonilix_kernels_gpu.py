@@ -178,7 +178,7 @@ def run_scan(ops, cuts, q, k, v, z, zb, coef, sign, beta, H, G, D, V, unit, q_sc
     return torch.cat(outs), state
 
 
-SCAN_SIZES = [(4, 2, 24, 10), (1, 1, 32, 48), (2, 2, 128, 16), (3, 1, 7, 5), (2, 1, 200, 8), (6, 3, 64, 64), (2, 2, 16, 130)]
+SCAN_SIZES = [(4, 2, 24, 10), (1, 1, 32, 48), (2, 2, 128, 16), (3, 1, 7, 5), (2, 1, 200, 8), (6, 3, 64, 64), (2, 2, 16, 130), (1, 1, 300, 6), (2, 1, 8, 3), (2, 2, 4, 70)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -214,6 +214,32 @@ def test_gated_linear_attention_over_steps(ops, dtype, H, G, D, V, tau):
         got, state = run_scan(ops, cuts, q, k, v, z, zb, coef, -1.0, None, H, G, D, V, False, D ** -0.5)
         close(got, want.reshape(T, H * V), dtype, f"outputs, portions {cuts[:4]}", tol=5e-5 if dtype == "float32" else 2e-2)
         close(state[1], S.transpose(1, 2), "float32", f"the slot's matrices, portions {cuts[:4]}", tol=5e-5)
+
+
+@pytest.mark.parametrize("H,G,D,V", [(4, 2, 24, 10), (2, 2, 128, 16), (1, 1, 300, 6)])
+def test_recurrences_take_decays_worked_out_by_the_low_rank_kernel(ops, H, G, D, V):
+    """The path the mixers take: the second half of the decay's low-rank pair hands on exp(-coef softplus(sign y))
+    itself, and the recurrence is told so (sign 0).  Long enough for several chunks."""
+    T, R = 150, 6
+    q, k, v, _, zb, beta = scan_inputs(H + D, T, H, G, D, V, "float32")
+    g = torch.Generator().manual_seed(9)
+    mid, w = torch.randn(T, R, generator=g), torch.randn(H * D, R, generator=g)
+    coef = torch.exp(torch.randn(H, generator=g) * 0.7)
+    y = mid.double() @ w.double().T + zb.double()
+    for sign, with_beta in ((1.0, True), (-1.0, False)):
+        dec = ops.lowrank_up(mid.to(DEV), w.to(DEV), zb.to(DEV), decay_coef=coef.to(DEV), decay_sign=sign)
+        gd = torch.exp(-coef.double()[None, :, None] * TP.softplus(sign * y).view(T, H, D))
+        close(dec, gd.reshape(T, H * D), "float32", "decays", tol=2e-6)
+        qd = q.double().view(T, G, D).repeat_interleave(H // G, 1)
+        kd = k.double().view(T, G, D).repeat_interleave(H // G, 1)
+        if with_beta:
+            want, _ = TP.delta_rule_scan(qd * 0.3, kd * 0.1, v.double().view(T, H, V), gd, torch.sigmoid(beta.double()))
+        else:
+            want, _ = TP.decayed_outer_scan(qd * 0.3, kd * 0.1, v.double().view(T, H, V), gd)
+        for cuts in ([T], [70, 1, 33, 46]):
+            got, _ = run_scan(ops, cuts, q, k * 0.1, v, dec.cpu(), None, coef, 0.0, beta if with_beta else None, H, G, D, V,
+                              False, 0.3)
+            close(got, want.reshape(T, H * V), "float32", f"sign {sign}, portions {cuts}", floor=0.1, tol=5e-5)
 
 
 def test_recurrence_keeps_one_early_write_for_hundreds_of_tokens(ops):
