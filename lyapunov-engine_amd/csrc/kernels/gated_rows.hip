@@ -27,33 +27,74 @@ __global__ __launch_bounds__(256) void group_rmsnorm_kernel(float* __restrict__ 
                                                             const float* __restrict__ scale,
                                                             const float* __restrict__ w, T* __restrict__ out,
                                                             const int32_t* __restrict__ rows, int H, int groups,
-                                                            float eps) {
-  extern __shared__ float s_group[];   // the row, then a float per wave
+                                                            float eps, int stage_w) {
+  extern __shared__ float s_group[];   // the row, a float per wave, then (stage_w) the norm's weights
   float* srow = s_group;
   float* scratch = s_group + H;
+  float* sw = s_group + H + 16;
   const int r = blockIdx.x;
   const size_t src = rows != nullptr ? static_cast<size_t>(rows[r]) : static_cast<size_t>(r);
   float* hrow = h + src * H;
-  for (int i = threadIdx.x; i < H; i += blockDim.x) {
-    float v = hrow[i];
-    if (delta != nullptr) {
-      float d = to_f32(delta[src * H + i]);
-      for (int p = 1; p < n_parts; ++p) d += to_f32(delta[p * part_stride + src * H + i]);
-      v += scale != nullptr ? d * scale[i] : d;
-      if (rows == nullptr) hrow[i] = v;
+  // eight values a thread at a time, their loads all issued before the first is used
+  constexpr int U = 8;
+  for (int i0 = threadIdx.x; i0 < H; i0 += U * blockDim.x) {
+    float hv[U], dv[U], sv[U], wv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * blockDim.x;
+      const bool in = i < H;
+      hv[u] = in ? hrow[i] : 0.f;
+      dv[u] = (in && delta != nullptr) ? to_f32(delta[src * H + i]) : 0.f;
+      sv[u] = (in && delta != nullptr && scale != nullptr) ? scale[i] : 1.f;
+      wv[u] = (in && stage_w && out != nullptr) ? w[i] : 0.f;
     }
-    srow[i] = v;
+    if (delta != nullptr) {
+      for (int p = 1; p < n_parts; ++p) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int i = i0 + u * blockDim.x;
+          if (i < H) dv[u] += to_f32(delta[p * part_stride + src * H + i]);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int i = i0 + u * blockDim.x;
+      if (i >= H) continue;
+      float v = hv[u];
+      if (delta != nullptr) {
+        v += dv[u] * sv[u];
+        if (rows == nullptr) hrow[i] = v;
+      }
+      srow[i] = v;
+      if (stage_w && out != nullptr) sw[i] = wv[u];
+    }
   }
   if (out == nullptr) return;
+  const float* wn = stage_w ? sw : w;
   const int gs = H / groups;
   T* orow = out + static_cast<size_t>(r) * H;
+  const int waves = blockDim.x / kWave;
+  if (groups >= waves) {
+    // a wave a group at a time: no workgroup-wide sums, and a group's sum does not depend on the others
+    __syncthreads();
+    const int lane = threadIdx.x % kWave;
+    for (int g = threadIdx.x / kWave; g < groups; g += waves) {
+      const float* sg = srow + g * gs;
+      float ss = 0.f;
+      for (int i = lane; i < gs; i += kWave) ss += sg[i] * sg[i];
+      const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(gs) + eps);
+      for (int i = lane; i < gs; i += kWave) orow[g * gs + i] = from_f32<T>(sg[i] * inv * wn[g * gs + i]);
+    }
+    return;
+  }
   for (int g = 0; g < groups; ++g) {
     float ss = 0.f;
     __syncthreads();
     for (int i = threadIdx.x; i < gs; i += blockDim.x) ss += srow[g * gs + i] * srow[g * gs + i];
     const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / static_cast<float>(gs) + eps);
     for (int i = threadIdx.x; i < gs; i += blockDim.x)
-      orow[g * gs + i] = from_f32<T>(srow[g * gs + i] * inv * w[g * gs + i]);
+      orow[g * gs + i] = from_f32<T>(srow[g * gs + i] * inv * wn[g * gs + i]);
   }
 }
 
@@ -173,12 +214,13 @@ int lyp_group_rmsnorm(float* h, const void* delta, int delta_dtype, int delta_pa
   LYP_REQUIRE(delta_parts == 0 || delta_dtype == kF32, "group_rmsnorm: partial sums are float");
   if (n_rows == 0) return 0;
   const int threads = H >= 1024 ? 256 : (H >= 256 ? 128 : 64);
-  const size_t lds = (static_cast<size_t>(H) + 16) * sizeof(float);
+  const int stage_w = (2 * static_cast<size_t>(H) + 16) * sizeof(float) <= 65536;
+  const size_t lds = (static_cast<size_t>(stage_w ? 2 * H : H) + 16) * sizeof(float);
   const int parts = delta_parts == 0 ? 1 : delta_parts;
 #define LYP_GN(TD, T)                                                                                              \
   group_rmsnorm_kernel<TD, T><<<n_rows, threads, lds, stream>>>(h, static_cast<const TD*>(delta), parts,           \
                                                                static_cast<size_t>(part_stride), scale, w,        \
-                                                               static_cast<T*>(out), rows, H, groups, eps)
+                                                               static_cast<T*>(out), rows, H, groups, eps, stage_w)
   const bool dbf = delta != nullptr && delta_dtype == kBF16;
   if (out_dtype == kBF16 && out != nullptr) {
     if (dbf) LYP_GN(bf16_t, bf16_t);

@@ -397,12 +397,24 @@ __global__ __launch_bounds__(kGroupedRows* kWave) void moe_route_grouped_kernel(
         we[j] = w + static_cast<size_t>(min(e0 + j, E - 1)) * K;   // past the last expert: worked out, not kept
       }
       if (vec_ok) {
-        for (int k = lane * 4; k < K; k += kWave * 4) {
-          const f32x4 xv = route_load4<T>(xr + k);
+        // four steps of the inner dimension at a time, their loads all issued before the first is used
+        constexpr int U = 4;
+        for (int k0 = lane * 4; k0 < K; k0 += kWave * 4 * U) {
+          f32x4 xv[U], wv[U][kRouteBlock];
 #pragma unroll
-          for (int j = 0; j < kRouteBlock; ++j) {
-            const f32x4 wv = *reinterpret_cast<const f32x4*>(we[j] + k);
-            acc[j] += xv[0] * wv[0] + xv[1] * wv[1] + xv[2] * wv[2] + xv[3] * wv[3];
+          for (int u = 0; u < U; ++u) {
+            const int k = k0 + u * kWave * 4;
+            const bool in = k < K;
+            xv[u] = in ? route_load4<T>(xr + k) : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < kRouteBlock; ++j)
+              wv[u][j] = in ? *reinterpret_cast<const f32x4*>(we[j] + k) : f32x4{0.f, 0.f, 0.f, 0.f};
+          }
+#pragma unroll
+          for (int u = 0; u < U; ++u) {
+#pragma unroll
+            for (int j = 0; j < kRouteBlock; ++j)
+              acc[j] += xv[u][0] * wv[u][j][0] + xv[u][1] * wv[u][j][1] + xv[u][2] * wv[u][j][2] + xv[u][3] * wv[u][j][3];
           }
         }
       } else {
