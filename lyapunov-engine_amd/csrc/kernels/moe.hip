@@ -376,6 +376,52 @@ __device__ __forceinline__ ArgMax wave_argmax(ArgMax m) {
   return m;
 }
 
+// One wave chooses for a row: c [E] choice scores (set to minus infinity as experts are chosen), sc [E] plain scores, both in LDS.
+__device__ __forceinline__ void choose_grouped(float* c, const float* sc, int lane, int row, int E, int top, int n_groups,
+                                               int keep, float scale, int32_t* __restrict__ idx, float* __restrict__ wgt) {
+  const int per = E / n_groups;
+  // a lane a group: the sum of its two largest choice scores (its one score for a group of one)
+  float gs = LYP_NEG_INF;
+  if (lane < n_groups) {
+    float a = LYP_NEG_INF, b = LYP_NEG_INF;
+    for (int i = 0; i < per; ++i) {
+      const float v = c[lane * per + i];
+      if (v > a) {
+        b = a;
+        a = v;
+      } else if (v > b) {
+        b = v;
+      }
+    }
+    gs = per > 1 ? a + b : a;
+  }
+  unsigned long long kept = 0ull;
+  bool mine_taken = lane >= n_groups;
+  for (int n = 0; n < keep; ++n) {
+    ArgMax m{mine_taken ? LYP_NEG_INF : gs, mine_taken ? 0x7fffffff : lane};
+    m = wave_argmax(m);
+    kept |= 1ull << m.i;
+    if (lane == m.i) mine_taken = true;
+  }
+  float total = 0.f;
+  int chosen = 0;   // lane n keeps the n-th choice
+  for (int n = 0; n < top; ++n) {
+    ArgMax m{LYP_NEG_INF, 0x7fffffff};
+    for (int e = lane; e < E; e += kWave)
+      if ((kept >> (e / per)) & 1ull) m = better(m, ArgMax{c[e], e});
+    m = wave_argmax(m);
+    if (lane == n) chosen = m.i;
+    if (lane == 0) c[m.i] = LYP_NEG_INF;
+    total += sc[m.i];
+    // the wave's lanes run together: the store above is seen by the next round's reads
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (lane < top) {
+    idx[static_cast<size_t>(row) * top + lane] = chosen;
+    wgt[static_cast<size_t>(row) * top + lane] = sc[chosen] / (total + 1e-20f) * scale;
+  }
+}
+
 template <typename T>
 __global__ __launch_bounds__(kGroupedRows* kWave) void moe_route_grouped_kernel(
     const T* __restrict__ x, int ldx, const float* __restrict__ w, const float* __restrict__ correction, int rows, int E,
@@ -437,48 +483,28 @@ __global__ __launch_bounds__(kGroupedRows* kWave) void moe_route_grouped_kernel(
   }
   __syncthreads();
   if (share != 0 || row >= rows) return;
-  float* c = s_choice[slot];
-  const int per = E / n_groups;
-  // a lane a group: the sum of its two largest choice scores (its one score for a group of one)
-  float gs = LYP_NEG_INF;
-  if (lane < n_groups) {
-    float a = LYP_NEG_INF, b = LYP_NEG_INF;
-    for (int i = 0; i < per; ++i) {
-      const float v = c[lane * per + i];
-      if (v > a) {
-        b = a;
-        a = v;
-      } else if (v > b) {
-        b = v;
-      }
-    }
-    gs = per > 1 ? a + b : a;
+  choose_grouped(s_choice[slot], s_score[slot], lane, row, E, top, n_groups, keep, scale, idx, wgt);
+}
+
+// The choice alone, from logits that the router's product kernel left as partial sums `part` [parts][rows][E]
+// (added up here in their order): a wave a row.
+__global__ __launch_bounds__(kGroupedRows* kWave) void moe_choose_grouped_kernel(
+    const float* __restrict__ part, int parts, const float* __restrict__ correction, int rows, int E, int top,
+    int n_groups, int keep, float scale, int32_t* __restrict__ idx, float* __restrict__ wgt) {
+  __shared__ float s_score[kGroupedRows][kMostExperts];
+  __shared__ float s_choice[kGroupedRows][kMostExperts];
+  const int lane = threadIdx.x % kWave, wave = threadIdx.x / kWave;
+  const int row = blockIdx.x * kGroupedRows + wave;
+  if (row >= rows) return;
+  for (int e = lane; e < E; e += kWave) {
+    float z = part[static_cast<size_t>(row) * E + e];
+    for (int p = 1; p < parts; ++p) z += part[(static_cast<size_t>(p) * rows + row) * E + e];
+    const float sg = 1.0f / (1.0f + expf(-z));
+    s_score[wave][e] = sg;
+    s_choice[wave][e] = sg + (correction != nullptr ? correction[e] : 0.f);
   }
-  unsigned long long kept = 0ull;
-  bool mine_taken = lane >= n_groups;
-  for (int n = 0; n < keep; ++n) {
-    ArgMax m{mine_taken ? LYP_NEG_INF : gs, mine_taken ? 0x7fffffff : lane};
-    m = wave_argmax(m);
-    kept |= 1ull << m.i;
-    if (lane == m.i) mine_taken = true;
-  }
-  float total = 0.f;
-  int chosen = 0;   // lane n keeps the n-th choice
-  for (int n = 0; n < top; ++n) {
-    ArgMax m{LYP_NEG_INF, 0x7fffffff};
-    for (int e = lane; e < E; e += kWave)
-      if ((kept >> (e / per)) & 1ull) m = better(m, ArgMax{c[e], e});
-    m = wave_argmax(m);
-    if (lane == n) chosen = m.i;
-    if (lane == 0) c[m.i] = LYP_NEG_INF;
-    total += s_score[slot][m.i];
-    // the wave's lanes run together: the store above is seen by the next round's reads
-    __builtin_amdgcn_wave_barrier();
-  }
-  if (lane < top) {
-    idx[static_cast<size_t>(row) * top + lane] = chosen;
-    wgt[static_cast<size_t>(row) * top + lane] = s_score[slot][chosen] / (total + 1e-20f) * scale;
-  }
+  __builtin_amdgcn_wave_barrier();
+  choose_grouped(s_choice[wave], s_score[wave], lane, row, E, top, n_groups, keep, scale, idx, wgt);
 }
 
 
@@ -901,6 +927,22 @@ int lyp_moe_route_grouped(const void* x, int ldx, int dtype, const float* w, con
   else
     LYP_REQUIRE(false, "moe_route_grouped: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("moe_route_grouped");
+  return 0;
+}
+
+// part float [parts][rows][E]: the router's logits as partial sums; the choice within groups as in lyp_moe_route_grouped.
+int lyp_moe_choose_grouped(const float* part, int parts, const float* correction, int rows, int E, int top, int n_groups,
+                           int keep, float scale, int32_t* idx, float* wgt, hipStream_t stream) {
+  LYP_REQUIRE(part != nullptr && parts >= 1 && rows >= 0 && E > 0 && E <= kMostExperts && top > 0 && top <= kMostTop,
+              "moe_choose_grouped: %d parts, %d rows, %d experts (at most %d), %d chosen (at most %d)", parts, rows, E,
+              kMostExperts, top, kMostTop);
+  LYP_REQUIRE(n_groups >= 1 && n_groups <= 64 && E % n_groups == 0 && keep >= 1 && keep <= n_groups &&
+                  keep * (E / n_groups) >= top,
+              "moe_choose_grouped: %d experts in %d groups of which %d are kept cannot give %d choices", E, n_groups, keep, top);
+  if (rows == 0) return 0;
+  moe_choose_grouped_kernel<<<(rows + kGroupedRows - 1) / kGroupedRows, kGroupedRows * kWave, 0, stream>>>(
+      part, parts, correction, rows, E, top, n_groups, keep, scale, idx, wgt);
+  LYP_LAUNCH_CHECK("moe_choose_grouped");
   return 0;
 }
 

@@ -149,6 +149,8 @@ def core() -> ctypes.CDLL:
                                            c_int, c_float, c_int, c_void_p]
         lib.lyp_lowrank_up.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                        c_void_p, c_float, c_int, c_void_p]
+        lib.lyp_moe_choose_grouped.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
+                                               c_void_p, c_void_p, c_void_p]
         lib.lyp_moe_route_grouped.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                               c_int, c_int, c_float, c_void_p, c_void_p, c_void_p]
         _core = lib
@@ -1507,11 +1509,14 @@ def moe_combine(y: torch.Tensor, plan: MoePlan, weights: torch.Tensor, rows: int
 
 
 def moe_route_grouped(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor | None, top: int, groups: int,
-                      keep: int, scale: float):
+                      keep: int, scale: float, on_matrix_cores: bool = True):
     """Sigmoid scores s = sigmoid(x @ router.T) in 32-bit (x [T, K] activations, router [E, K] float); the
     choice goes by s + correction among the experts of the ``keep`` best of ``groups`` equal groups of
     neighbours (a group's score: the sum of its two largest choice scores), the weights are the chosen
-    experts' s over their sum, times ``scale``.  -> (experts int32 [T, top], weights float [T, top])."""
+    experts' s over their sum, times ``scale``.  -> (experts int32 [T, top], weights float [T, top]).
+    The logits come from the router's product kernel on the float matrix instruction (workgroups share
+    the inner dimension and leave partial sums, which the choice's kernel adds up in their order);
+    ``on_matrix_cores=False``: product and choice in one kernel of plain float sums, a wave a row."""
     _rows_view(x, "moe_route_grouped")
     _dev(router, correction)
     _f32(router, correction)
@@ -1522,8 +1527,16 @@ def moe_route_grouped(x: torch.Tensor, router: torch.Tensor, correction: torch.T
     idx = torch.empty((T, top), dtype=torch.int32, device=x.device)
     wgt = torch.empty((T, top), dtype=torch.float32, device=x.device)
     lib = core()
-    _check(lib.lyp_moe_route_grouped(_p(x), x.stride(0), _code(x.dtype), _p(router), _p(correction), T, E, K, top,
-                                     int(groups), int(keep), float(scale), _p(idx), _p(wgt), _stream()), lib)
+    if not on_matrix_cores:
+        _check(lib.lyp_moe_route_grouped(_p(x), x.stride(0), _code(x.dtype), _p(router), _p(correction), T, E, K, top,
+                                         int(groups), int(keep), float(scale), _p(idx), _p(wgt), _stream()), lib)
+        return idx, wgt
+    splits = max(2, lib.lyp_moe_route_splits(T, K))      # two shares at the least: the product then leaves its sums
+    part = torch.empty((splits, T, E), dtype=torch.float32, device=x.device)
+    _check(lib.lyp_moe_route_fused(_p(x), x.stride(0), _code(x.dtype), _p(router), None, T, E, K, top, _p(idx), _p(wgt), -1,
+                                   _p(part), splits, 0, _stream()), lib)
+    _check(lib.lyp_moe_choose_grouped(_p(part), splits, _p(correction), T, E, top, int(groups), int(keep), float(scale),
+                                      _p(idx), _p(wgt), _stream()), lib)
     return idx, wgt
 
 

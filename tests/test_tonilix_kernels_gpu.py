@@ -385,16 +385,18 @@ ROUTERS = [dict(experts=6, top=2, scale=1.5, groups=dict(count=3, keep=2)), dict
            dict(experts=12, top=4, scale=1.0, groups=dict(count=1, keep=1)), dict(experts=256, top=8, scale=2.5, groups=dict(count=8, keep=4))]
 
 
+@pytest.mark.parametrize("cores", [True, False], ids=["matrix cores", "plain sums"])
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("r", ROUTERS, ids=lambda r: f"{r['top']}of{r['experts']}in{r['groups']['keep']}of{r['groups']['count']}")
-def test_router_chooses_within_the_best_groups(ops, dtype, r):
+def test_router_chooses_within_the_best_groups(ops, dtype, r, cores):
     E, top = r["experts"], r["top"]
     T, K = 50, 40
     g = torch.Generator().manual_seed(E)
     x = torch.randn(T, K, generator=g).to(tdt(dtype))
     W = torch.randn(E, K, generator=g) * 0.5
     corr = torch.randn(E, generator=g) * 0.6 - 0.8          # many choice scores are negative
-    idx, wgt = ops.moe_route_grouped(x.to(DEV), W.to(DEV), corr.to(DEV), top, r["groups"]["count"], r["groups"]["keep"], r["scale"])
+    idx, wgt = ops.moe_route_grouped(x.to(DEV), W.to(DEV), corr.to(DEV), top, r["groups"]["count"], r["groups"]["keep"], r["scale"],
+                                     on_matrix_cores=cores)
     s = torch.sigmoid(x.double() @ W.double().T)
     margins = []
     chosen, weights = TP.choose_experts(s, corr.double(), r, margins)
