@@ -45,10 +45,15 @@ __device__ __forceinline__ float scan_dpp(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
 }
 __device__ __forceinline__ float group_sum(float v, int L) {
-  if (L > 1) v += scan_dpp<0xB1>(v);    // neighbours: lanes 1 0 3 2 of every four
-  if (L > 2) v += scan_dpp<0x4E>(v);    // lanes 2 3 0 1 of every four
-  if (L > 4) v += scan_dpp<0x141>(v);   // every eight mirrored
-  if (L > 8) v += scan_dpp<0x140>(v);   // every sixteen mirrored
+  // every stage is worked out and taken or not by a select: no branches in the walk over the tokens
+  float t = v + scan_dpp<0xB1>(v);    // neighbours: lanes 1 0 3 2 of every four
+  v = L > 1 ? t : v;
+  t = v + scan_dpp<0x4E>(v);          // lanes 2 3 0 1 of every four
+  v = L > 2 ? t : v;
+  t = v + scan_dpp<0x141>(v);         // every eight mirrored
+  v = L > 4 ? t : v;
+  t = v + scan_dpp<0x140>(v);         // every sixteen mirrored
+  v = L > 8 ? t : v;
   return v;
 }
 
@@ -80,6 +85,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
   float* sfq = sb + chunk;                     // [chunk]       what a query is multiplied by (unit length, the constant)
   float* sfk = sfq + chunk;                    // [chunk]       what a key is multiplied by
   float* sqk = sfk + chunk;                    // [chunk]       query . key, as they come
+  float* so = sqk + chunk;                     // [chunk][cpb]  the tokens' outputs, written out a chunk at a time
   const int b = blockIdx.z, h = blockIdx.y;
   const int q0 = q_start[b], n = q_start[b + 1] - q0;
   if (n <= 0) return;
@@ -240,7 +246,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
 #pragma unroll
         for (int e = 0; e < 4; ++e) S[4 * i + e] += k_[i][e] * u_;
       }
-      if (l == 0 && col < V) out[static_cast<size_t>(q0 + c0 + j) * ldo + h * V + col] = fq_ * (p + qk_ * u_);
+      so[(j << cpb_shift) + cl] = fq_ * (p + qk_ * u_);   // all lanes of the column hold it: no branch
     };
     // two tokens a round, their operands in two sets of registers in turn
     read(0, g4, q4, k4, fk, fq, qk, u, bt);
@@ -253,6 +259,10 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
       }
     }
     __syncthreads();   // the chunk's staging is read to the end before the next overwrites it
+    for (int idx = tid; idx < (cn << cpb_shift); idx += blockDim.x) {
+      const int j = idx >> cpb_shift, c = blockIdx.x * cpb + (idx & (cpb - 1));
+      if (c < V) out[static_cast<size_t>(q0 + c0 + j) * ldo + h * V + c] = so[idx];
+    }
   }
   if (col < V) {
 #pragma unroll
@@ -363,8 +373,10 @@ int lyp_linear_scan(const void* q, int ldq, const void* k, int ldk, const void* 
   dim3 grid((V + cpb - 1) / cpb, H, B);
   // few rows a request (single tokens, short portions): a short chunk, so that many workgroups fit a compute unit
   const bool brief = rows < 16LL * B;
-  const int chunk = brief ? (rows <= B ? 2 : std::min(8, scan_chunk(L * dpl))) : scan_chunk(L * dpl);
-  const size_t lds = static_cast<size_t>(chunk) * (3 * (L * dpl + kScanPad) + cpb + 4) * sizeof(float);
+  int chunk = brief ? (rows <= B ? 2 : std::min(8, scan_chunk(L * dpl))) : scan_chunk(L * dpl);
+  const size_t per_token = (3 * (L * dpl + kScanPad) + 2 * cpb + 4) * sizeof(float);
+  while (chunk > 1 && chunk * per_token > 65536) chunk /= 2;
+  const size_t lds = chunk * per_token;
 #define LYP_SCAN_S(T, DPLV, DEL, ST)                                                                                \
   linear_scan_kernel<T, DPLV, DEL, ST><<<grid, threads, lds, stream>>>(                                               \
       static_cast<const T*>(q), ldq, static_cast<const T*>(k), ldk, static_cast<const T*>(v), ldv, z, ldz, zbias,   \
