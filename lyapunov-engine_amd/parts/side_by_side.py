@@ -34,6 +34,9 @@ class SideBySide(Mixer):
             if getattr(self.left, what)() is not None and getattr(self.right, what)() is not None:
                 raise ValueError(f"two mixers side by side: only one of them may have a {what}")
         self.graph_safe = self.left.graph_safe and self.right.graph_safe
+        # a left mixer that can leave its output bias to us: the weighted sum's kernel adds it
+        if hasattr(self.left, "defer_bias"):
+            self.left.defer_bias = True
 
     def children(self):
         return {self.names["left"]: self.left, self.names["right"]: self.right}
@@ -69,4 +72,5 @@ class SideBySide(Mixer):
     def forward(self, ctx: StepContext, x, cache: LayerCache):
         a = self._tensor(self.left.forward(ctx, x, self._for_child(cache, "left")))
         b = self._tensor(self.right.forward(ctx, x, self._for_child(cache, "right")))
-        return ops.weighted_sum(a, self.left_scale, b, self.right_scale)
+        bias = getattr(self.left, "o_bias_f", None) if getattr(self.left, "defer_bias", False) else None
+        return ops.weighted_sum(a, self.left_scale, b, self.right_scale, bias)

@@ -50,6 +50,8 @@ class TemperedAttention(Mixer):
         self.matrix_cores = self.dim == self.vdim and self.dim % 16 == 0 and self.dim <= 256
         self.in_proj = self.in_bias = self.o_proj = self.o_bias = None
         self.in_bias_f = self.o_bias_f = None
+        # True: ``forward`` leaves the output projection's bias to its caller (``o_bias_f``), who adds it in a kernel of its own
+        self.defer_bias = False
 
     def weight_specs(self):
         n, H, G, C = self.names, self.num_heads, self.num_kv_heads, self.hidden_size
@@ -109,6 +111,6 @@ class TemperedAttention(Mixer):
             at = (H + G) * self.dim + G * self.vdim
             ops.gate_mul(out, pre[:, at:at + H * self.vdim], "sigmoid")
         y = ops.linear(out, self.o_proj, out_dtype=torch.float32)
-        if self.o_bias_f is not None:
+        if self.o_bias_f is not None and not self.defer_bias:
             ops.add_row(y, self.o_bias_f)
         return y
