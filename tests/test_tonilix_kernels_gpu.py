@@ -44,7 +44,7 @@ def ops():
 
 # ------------------------------------------------------------ norm in groups
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,groups", [(72, 3), (64, 1), (128, 4), (100, 5), (2048, 8), (40, 40)])
+@pytest.mark.parametrize("H,groups", [(72, 3), (64, 1), (128, 4), (100, 5), (2048, 8), (40, 40), (2048, 2), (512, 1), (1024, 1), (9000, 3)])
 def test_group_norm_adds_the_scaled_branch_first(ops, dtype, H, groups):
     T = 11
     g = torch.Generator().manual_seed(H + groups)
