@@ -148,11 +148,11 @@ __global__ void glu_act_vec_kernel(const T* __restrict__ gu, T* __restrict__ out
 
 template <typename TG, typename T>
 __global__ void gate_mul_kernel(T* __restrict__ x, const TG* __restrict__ gate, int ldg, int N, size_t total,
-                                int kind) {
+                                int kind, int per) {
   const size_t idx = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t t = idx / N, c = idx % N;
-  const float g = to_f32(gate[t * ldg + c]);
+  const float g = to_f32(gate[t * ldg + c / per]);   // one gate value for `per` neighbours (a head's values)
   const float s = 1.0f / (1.0f + expf(-g));
   x[idx] = from_f32<T>(to_f32(x[idx]) * (kind == 1 ? g * s : s));
 }
@@ -272,20 +272,22 @@ int lyp_glu_act(const void* gate_up, void* out, int dtype, int T, int I, int act
   return 0;
 }
 
-// x [T, N] of dtype; gate [T, >= N] (ldg apart) float (gate_dtype kF32) or of x's type; kind 0 sigmoid, 1 silu.
-int lyp_gate_mul(void* x, int dtype, const void* gate, int ldg, int gate_dtype, int T, int N, int kind,
+// x [T, N] of dtype; gate [T, >= N / per] (ldg apart) float (gate_dtype kF32) or of x's type, one value for
+// every `per` neighbouring values of x; kind 0 sigmoid, 1 silu.
+int lyp_gate_mul(void* x, int dtype, const void* gate, int ldg, int gate_dtype, int T, int N, int kind, int per,
                  hipStream_t stream) {
-  LYP_REQUIRE(T >= 0 && N > 0 && ldg >= N && (kind == 0 || kind == 1), "gate_mul: T=%d N=%d ldg=%d kind=%d", T, N, ldg, kind);
+  LYP_REQUIRE(T >= 0 && N > 0 && per > 0 && N % per == 0 && ldg >= N / per && (kind == 0 || kind == 1),
+              "gate_mul: T=%d N=%d ldg=%d kind=%d per=%d", T, N, ldg, kind, per);
   LYP_REQUIRE(gate_dtype == kF32 || gate_dtype == dtype, "gate_mul: the gate is float or of x's type");
   if (T == 0) return 0;
   const size_t total = static_cast<size_t>(T) * N;
   const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
   if (dtype == kF32)
-    gate_mul_kernel<float, float><<<blocks, 256, 0, stream>>>(static_cast<float*>(x), static_cast<const float*>(gate), ldg, N, total, kind);
+    gate_mul_kernel<float, float><<<blocks, 256, 0, stream>>>(static_cast<float*>(x), static_cast<const float*>(gate), ldg, N, total, kind, per);
   else if (dtype == kBF16 && gate_dtype == kF32)
-    gate_mul_kernel<float, bf16_t><<<blocks, 256, 0, stream>>>(static_cast<bf16_t*>(x), static_cast<const float*>(gate), ldg, N, total, kind);
+    gate_mul_kernel<float, bf16_t><<<blocks, 256, 0, stream>>>(static_cast<bf16_t*>(x), static_cast<const float*>(gate), ldg, N, total, kind, per);
   else if (dtype == kBF16)
-    gate_mul_kernel<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>(static_cast<bf16_t*>(x), static_cast<const bf16_t*>(gate), ldg, N, total, kind);
+    gate_mul_kernel<bf16_t, bf16_t><<<blocks, 256, 0, stream>>>(static_cast<bf16_t*>(x), static_cast<const bf16_t*>(gate), ldg, N, total, kind, per);
   else
     LYP_REQUIRE(false, "gate_mul: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("gate_mul");

@@ -5,9 +5,14 @@
 //   gated delta rule          S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);
 //                             S <- S + k_t u^T                                 o_t = S^T q_t
 //
+//   bonus for the current token   o_t = (S + diag(u) k_t v_t^T)^T q_t;  S <- diag(g_t) S + k_t v_t^T
+//                                 (the output reads the state before the token's decay and write)
+//
 // with a decay per head and key channel, g = exp(-coef_head * softplus(sign * (z + bias))), which
 // covers exp(-A softplus(z + b)) (sign +1, coef A) and sigmoid(z + b)^(1/tau) (sign -1, coef 1/tau);
-// sign 0 says that z holds the decays themselves (lowrank_up works them out on its way).
+// sign 0 says that z holds the decays themselves (lowrank_up works them out on its way).  One decay
+// per head (z [rows, heads]) is taken for all of the head's key channels; the softplus is then a step
+// size that may also multiply the token's key (S <- g S + step k v^T: a discretised state space).
 // Queries and keys may be made unit vectors per head first (x / sqrt(sum x^2 + 1e-6)); queries
 // take a constant factor.  Decays, unit vectors, gates, sums and the state are 32-bit; q, k, v come
 // in the activations' type.
@@ -64,13 +69,16 @@ __device__ __forceinline__ float group_sum(float v, int L) {
 // STAGE: keys, queries and decays a thread fetches in one round (and half as many values): 16 for steps
 // of long portions, 4 for steps of single tokens and short portions, which then need few registers
 // and many workgroups fit a compute unit.
-template <typename T, int DPL, bool DELTA, int STAGE>
+// MODE 0: decayed outer products, 1: the delta rule, 2: the bonus form.
+template <typename T, int DPL, int MODE, int STAGE>
 __global__ __launch_bounds__(256) void linear_scan_kernel(
     const T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, const T* __restrict__ v, int ldv,
     const float* __restrict__ z, int ldz, const float* __restrict__ zbias, const float* __restrict__ coef, float sign,
     const T* __restrict__ beta, int ldb, float* __restrict__ state, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, float* __restrict__ out, int ldo, int H,
-    int G, int D, int V, int L, int unit, float q_scale, int chunk) {
+    int G, int D, int V, int L, int unit, float q_scale, int chunk, const float* __restrict__ bonus, int z_per_head,
+    int key_step) {
+  constexpr bool DELTA = MODE == 1, PRE = MODE == 2;
   extern __shared__ __attribute__((aligned(16))) float s_scan[];
   const int Dp = L * DPL;                      // key channels with the padding: a power of two
   const int ld = Dp + kScanPad;
@@ -86,6 +94,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
   float* sfk = sfq + chunk;                    // [chunk]       what a key is multiplied by
   float* sqk = sfk + chunk;                    // [chunk]       query . key, as they come
   float* so = sqk + chunk;                     // [chunk][cpb]  the tokens' outputs, written out a chunk at a time
+  float* sbn = so + chunk * cpb;               // [Dp]          the head's bonus, laid out as a staged key (the bonus form only)
   const int b = blockIdx.z, h = blockIdx.y;
   const int q0 = q_start[b], n = q_start[b + 1] - q0;
   if (n <= 0) return;
@@ -123,7 +132,7 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
         const size_t row = static_cast<size_t>(q0 + c0 + j);
         rq[u] = q[row * ldq + kvh * D + d];
         rk[u] = k[row * ldk + kvh * D + d];
-        rz[u] = z[row * ldz + h * D + d];
+        rz[u] = z[row * ldz + (z_per_head ? h : h * D + d)];
       }
     }
   };
@@ -143,7 +152,9 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
       const int j = idx >> dp_shift, d = idx & (Dp - 1);
       if (j < cn) {
         float gg = 1.f;
-        if (d < D) gg = sign == 0.f ? rz[u] : expf(-a_h * scan_softplus(sign * (rz[u] + (zbias != nullptr ? zbias[h * D + d] : 0.f))));
+        if (d < D)
+          gg = sign == 0.f ? rz[u]
+                           : expf(-a_h * scan_softplus(sign * (rz[u] + (zbias != nullptr ? zbias[z_per_head ? h : h * D + d] : 0.f))));
         // a lane's channels four by four in planes, so that a plane's read takes neighbouring lanes to neighbouring words
         const int at = j * ld + ((((d & (DPL - 1)) >> 2) << (l_shift + 2)) | ((d / DPL) << 2) | (d & 3));
         sq[at] = to_f32(rq[u]);
@@ -163,6 +174,10 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
   if (ahead) {
     fetch(0, min(chunk, n), 0);
     fetch_values(0, min(chunk, n));
+  }
+  if constexpr (PRE) {
+    for (int d = tid; d < Dp; d += blockDim.x)
+      sbn[(((d & (DPL - 1)) >> 2) << (l_shift + 2)) | ((d / DPL) << 2) | (d & 3)] = d < D ? bonus[h * D + d] : 0.f;
   }
 
   for (int c0 = 0; c0 < n; c0 += chunk) {
@@ -190,14 +205,22 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
         const f32x4 k4 = *reinterpret_cast<const f32x4*>(sk + j * ld + 4 * f);
         ssq += q4[0] * q4[0] + q4[1] * q4[1] + q4[2] * q4[2] + q4[3] * q4[3];
         ssk += k4[0] * k4[0] + k4[1] * k4[1] + k4[2] * k4[2] + k4[3] * k4[3];
-        sqkv += q4[0] * k4[0] + q4[1] * k4[1] + q4[2] * k4[2] + q4[3] * k4[3];
+        if constexpr (PRE) {
+          const f32x4 b4 = *reinterpret_cast<const f32x4*>(sbn + 4 * f);
+          sqkv += q4[0] * k4[0] * b4[0] + q4[1] * k4[1] * b4[1] + q4[2] * k4[2] * b4[2] + q4[3] * k4[3] * b4[3];
+        } else {
+          sqkv += q4[0] * k4[0] + q4[1] * k4[1] + q4[2] * k4[2] + q4[3] * k4[3];
+        }
       }
       ssq = group_sum(ssq, 4);
       ssk = group_sum(ssk, 4);
       sqkv = group_sum(sqkv, 4);
       if (tid % 4 == 0) {
         sfq[j] = unit ? q_scale / sqrtf(ssq + 1e-6f) : q_scale;
-        sfk[j] = unit ? 1.0f / sqrtf(ssk + 1e-6f) : 1.f;
+        float fkey = unit ? 1.0f / sqrtf(ssk + 1e-6f) : 1.f;
+        if (key_step)   // the step size: the softplus inside the head's decay
+          fkey *= scan_softplus(sign * (z[static_cast<size_t>(q0 + c0 + j) * ldz + h] + (zbias != nullptr ? zbias[h] : 0.f)));
+        sfk[j] = fkey;
         sqk[j] = sqkv;
       }
     }
@@ -229,14 +252,20 @@ __global__ __launch_bounds__(256) void linear_scan_kernel(
       float r0 = 0.f, r1 = 0.f, p0 = 0.f, p1 = 0.f;
 #pragma unroll
       for (int i = 0; i < DPL / 4; ++i) {
+        if constexpr (PRE) {   // the output reads the state as the token found it
+          p0 += S[4 * i] * q_[i][0] + S[4 * i + 2] * q_[i][2];
+          p1 += S[4 * i + 1] * q_[i][1] + S[4 * i + 3] * q_[i][3];
+        }
 #pragma unroll
         for (int e = 0; e < 4; ++e) S[4 * i + e] *= g_[i][e];
         if constexpr (DELTA) {
           r0 += S[4 * i] * k_[i][0] + S[4 * i + 2] * k_[i][2];
           r1 += S[4 * i + 1] * k_[i][1] + S[4 * i + 3] * k_[i][3];
         }
-        p0 += S[4 * i] * q_[i][0] + S[4 * i + 2] * q_[i][2];
-        p1 += S[4 * i + 1] * q_[i][1] + S[4 * i + 3] * q_[i][3];
+        if constexpr (!PRE) {
+          p0 += S[4 * i] * q_[i][0] + S[4 * i + 2] * q_[i][2];
+          p1 += S[4 * i + 1] * q_[i][1] + S[4 * i + 3] * q_[i][3];
+        }
       }
       const float p = group_sum(p0 + p1, L);
       if constexpr (DELTA) u_ = bt_ * (u_ - fk_ * group_sum(r0 + r1, L));
@@ -277,7 +306,7 @@ enum GateKind : int { kGateSigmoid = 0, kGateSilu = 1 };
 template <typename TG, typename T>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, const float* __restrict__ w,
                                                              const TG* __restrict__ gate, int ldg, T* __restrict__ out,
-                                                             int rows, int H, int V, float eps, int kind) {
+                                                             int rows, int H, int V, float eps, int kind, int w_per_head) {
   const int item = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
   if (item >= rows * H) return;
   const int t = item / H, h = item % H, lane = threadIdx.x % kWave;
@@ -287,6 +316,7 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   const float inv = 1.0f / sqrtf(wave_sum(ss) / static_cast<float>(V) + eps);
   const TG* grow = gate + static_cast<size_t>(t) * ldg + h * V;
   T* dst = out + (static_cast<size_t>(t) * H + h) * V;
+  if (w_per_head) w += h * V;
   for (int c = lane; c < V; c += kWave) {
     const float g = to_f32(grow[c]);
     const float s = scan_sigmoid(g);
@@ -300,7 +330,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void lowrank_up_kernel(const T* __restrict__ mid, int ldm, const float* __restrict__ w,
                                                          const float* __restrict__ bias, float* __restrict__ out,
                                                          int rows, int N, int R, const float* __restrict__ coef,
-                                                         float sign, int per_head) {
+                                                         float sign, int per_head, int mid_tanh, int double_exp) {
   const int n = blockIdx.x * blockDim.x + threadIdx.x;
   const int t0 = blockIdx.y * kLowRows;
   if (n >= N) return;
@@ -313,13 +343,17 @@ __global__ __launch_bounds__(256) void lowrank_up_kernel(const T* __restrict__ m
     const float x = wr[r];
 #pragma unroll
     for (int j = 0; j < kLowRows; ++j)
-      if (t0 + j < rows) acc[j] += x * to_f32(mid[static_cast<size_t>(t0 + j) * ldm + r]);
+      if (t0 + j < rows) {
+        const float m = to_f32(mid[static_cast<size_t>(t0 + j) * ldm + r]);
+        acc[j] += x * (mid_tanh ? tanhf(m) : m);
+      }
   }
   const float a = coef != nullptr ? coef[n / per_head] : 0.f;
 #pragma unroll
   for (int j = 0; j < kLowRows; ++j)
     if (t0 + j < rows)
-      out[static_cast<size_t>(t0 + j) * N + n] = coef != nullptr ? expf(-a * scan_softplus(sign * acc[j])) : acc[j];
+      out[static_cast<size_t>(t0 + j) * N + n] = double_exp ? expf(-expf(acc[j]))
+                                                 : (coef != nullptr ? expf(-a * scan_softplus(sign * acc[j])) : acc[j]);
 }
 
 }  // namespace lyp
@@ -345,18 +379,21 @@ int lyp_linear_scan_lanes(int D) {
 }
 
 // q, k [rows, >= G*D] and v [rows, >= H*V] of dtype, rows ldq / ldk / ldv apart; z float [rows, >= H*D] (ldz apart);
-// zbias float [H*D] or null; coef float [H]; rows: all requests' rows together; beta [rows, >= H] of dtype (ldb apart; the delta rule only: delta != 0);
+// zbias float [H*D] or null (z_per_head: z [rows, >= H], zbias [H]; key_step: the key is multiplied by the softplus);
+// bonus float [H*D] or null (the bonus form); coef float [H]; rows: all requests' rows together; beta [rows, >= H] of dtype (ldb apart; the delta rule only: delta != 0);
 // state float [slots, H, V, D]; out float [rows, >= H*V] (ldo apart).  Request b owns rows q_start[b] .. q_start[b+1].
 int lyp_linear_scan(const void* q, int ldq, const void* k, int ldk, const void* v, int ldv, int dtype, const float* z,
                     int ldz, const float* zbias, const float* coef, float sign, const void* beta, int ldb,
                     float* state, const int32_t* q_start, const int32_t* positions, const int32_t* slots, float* out,
                     int ldo, int rows, int B, int H, int G, int D, int V, int delta, int unit, float q_scale,
-                    hipStream_t stream) {
+                    const float* bonus, int z_per_head, int key_step, hipStream_t stream) {
   LYP_REQUIRE(B > 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && V > 0, "linear_scan: B=%d H=%d G=%d D=%d V=%d", B, H, G,
               D, V);
   const int L = lyp_linear_scan_lanes(D);
   LYP_REQUIRE(L > 0 && L <= 16, "linear_scan: key heads of up to 512 values, not %d", D);
-  LYP_REQUIRE(ldq >= G * D && ldk >= G * D && ldv >= H * V && ldz >= H * D && ldo >= H * V && (!delta || ldb >= H),
+  LYP_REQUIRE(!(delta && bonus != nullptr), "linear_scan: the delta rule has no bonus form");
+  LYP_REQUIRE(!key_step || (z_per_head && sign != 0.f), "linear_scan: a step size comes with one decay per head, worked out here");
+  LYP_REQUIRE(ldq >= G * D && ldk >= G * D && ldv >= H * V && ldz >= (z_per_head ? H : H * D) && ldo >= H * V && (!delta || ldb >= H),
               "linear_scan: rows too short for %d/%d heads of %d/%d", H, G, D, V);
   LYP_REQUIRE(!delta || beta != nullptr, "linear_scan: the delta rule needs beta");
   LYP_REQUIRE(H <= 65535 && B <= 65535, "linear_scan: too many heads or requests for one launch");
@@ -375,45 +412,46 @@ int lyp_linear_scan(const void* q, int ldq, const void* k, int ldk, const void* 
   const bool brief = rows < 16LL * B;
   int chunk = brief ? (rows <= B ? 2 : std::min(8, scan_chunk(L * dpl))) : scan_chunk(L * dpl);
   const size_t per_token = (3 * (L * dpl + kScanPad) + 2 * cpb + 4) * sizeof(float);
-  while (chunk > 1 && chunk * per_token > 65536) chunk /= 2;
-  const size_t lds = chunk * per_token;
+  while (chunk > 1 && chunk * per_token > 65536 - 2048) chunk /= 2;
+  const size_t lds = chunk * per_token + (bonus != nullptr ? L * dpl * sizeof(float) : 0);
+  const int mode = delta ? 1 : (bonus != nullptr ? 2 : 0);
 #define LYP_SCAN_S(T, DPLV, DEL, ST)                                                                                \
   linear_scan_kernel<T, DPLV, DEL, ST><<<grid, threads, lds, stream>>>(                                               \
       static_cast<const T*>(q), ldq, static_cast<const T*>(k), ldk, static_cast<const T*>(v), ldv, z, ldz, zbias,   \
       coef, sign, static_cast<const T*>(beta), ldb, state, q_start, positions, slots, out, ldo, H, G, D, V, L, unit, \
-      q_scale, chunk)
+      q_scale, chunk, bonus, z_per_head, key_step)
 #define LYP_SCAN(T, DPLV, DEL)              \
   do {                                      \
     if (brief) LYP_SCAN_S(T, DPLV, DEL, 4); \
     else LYP_SCAN_S(T, DPLV, DEL, 16);      \
   } while (0)
+#define LYP_SCAN_M(T, DPLV)                    \
+  do {                                         \
+    if (mode == 1) LYP_SCAN(T, DPLV, 1);       \
+    else if (mode == 2) LYP_SCAN(T, DPLV, 2);  \
+    else LYP_SCAN(T, DPLV, 0);                 \
+  } while (0)
 #define LYP_SCAN_T(T)                          \
   do {                                         \
-    if (dpl == 8) {                            \
-      if (delta) LYP_SCAN(T, 8, true);         \
-      else LYP_SCAN(T, 8, false);              \
-    } else if (dpl == 16) {                    \
-      if (delta) LYP_SCAN(T, 16, true);        \
-      else LYP_SCAN(T, 16, false);             \
-    } else {                                   \
-      if (delta) LYP_SCAN(T, 32, true);        \
-      else LYP_SCAN(T, 32, false);             \
-    }                                          \
+    if (dpl == 8) LYP_SCAN_M(T, 8);            \
+    else if (dpl == 16) LYP_SCAN_M(T, 16);     \
+    else LYP_SCAN_M(T, 32);                    \
   } while (0)
   if (dtype == kF32) LYP_SCAN_T(float);
   else if (dtype == kBF16) LYP_SCAN_T(bf16_t);
   else LYP_REQUIRE(false, "linear_scan: unknown dtype %d", dtype);
 #undef LYP_SCAN_T
+#undef LYP_SCAN_M
 #undef LYP_SCAN
 #undef LYP_SCAN_S
   LYP_LAUNCH_CHECK("linear_scan");
   return 0;
 }
 
-// o float [rows, H*V]; w float [V]; gate [rows, >= H*V] (ldg apart) float (gate_dtype kF32) or of out's type;
+// o float [rows, H*V]; w float [V] (w_per_head: [H*V], every head its own); gate [rows, >= H*V] (ldg apart) float (gate_dtype kF32) or of out's type;
 // out [rows, H*V] of out_dtype.  kind: 0 sigmoid(gate), 1 silu(gate).
 int lyp_head_norm_gate(const float* o, const float* w, const void* gate, int ldg, int gate_dtype, void* out,
-                       int out_dtype, int rows, int H, int V, float eps, int kind, hipStream_t stream) {
+                       int out_dtype, int rows, int H, int V, float eps, int kind, int w_per_head, hipStream_t stream) {
   LYP_REQUIRE(rows >= 0 && H > 0 && V > 0 && ldg >= H * V && (kind == kGateSigmoid || kind == kGateSilu),
               "head_norm_gate: rows=%d H=%d V=%d ldg=%d kind=%d", rows, H, V, ldg, kind);
   LYP_REQUIRE(gate_dtype == kF32 || gate_dtype == out_dtype, "head_norm_gate: the gate is float or of the output's type");
@@ -422,7 +460,7 @@ int lyp_head_norm_gate(const float* o, const float* w, const void* gate, int ldg
   const int blocks = static_cast<int>((items + 3) / 4);
 #define LYP_HNG(TG, T)                                                                                              \
   head_norm_gate_kernel<TG, T><<<blocks, 256, 0, stream>>>(o, w, static_cast<const TG*>(gate), ldg,                 \
-                                                           static_cast<T*>(out), rows, H, V, eps, kind)
+                                                           static_cast<T*>(out), rows, H, V, eps, kind, w_per_head)
   if (out_dtype == kF32) LYP_HNG(float, float);
   else if (out_dtype == kBF16 && gate_dtype == kF32) LYP_HNG(float, bf16_t);
   else if (out_dtype == kBF16) LYP_HNG(bf16_t, bf16_t);
@@ -434,8 +472,9 @@ int lyp_head_norm_gate(const float* o, const float* w, const void* gate, int ldg
 
 // mid [rows, >= R] of dtype (ldm apart); w float [N, R]; bias float [N] or null; out float [rows, N].
 // coef float [N / per_head] or null: the result y becomes the decay exp(-coef[n / per_head] * softplus(sign * y)).
+// mid_tanh: the inner values pass tanh first; double_exp: the result y becomes the decay exp(-exp(y)).
 int lyp_lowrank_up(const void* mid, int ldm, int dtype, const float* w, const float* bias, float* out, int rows, int N,
-                   int R, const float* coef, float sign, int per_head, hipStream_t stream) {
+                   int R, const float* coef, float sign, int per_head, int mid_tanh, int double_exp, hipStream_t stream) {
   LYP_REQUIRE(coef == nullptr || (per_head > 0 && N % per_head == 0), "lowrank_up: %d values in heads of %d", N, per_head);
   LYP_REQUIRE(rows >= 0 && N > 0 && R > 0 && ldm >= R, "lowrank_up: rows=%d N=%d R=%d ldm=%d", rows, N, R, ldm);
   if (rows == 0) return 0;
@@ -443,9 +482,9 @@ int lyp_lowrank_up(const void* mid, int ldm, int dtype, const float* w, const fl
   dim3 grid((N + threads - 1) / threads, (rows + kLowRows - 1) / kLowRows);
   LYP_REQUIRE(grid.y <= 65535, "lowrank_up: too many rows for one launch");
   if (dtype == kF32)
-    lowrank_up_kernel<float><<<grid, threads, 0, stream>>>(static_cast<const float*>(mid), ldm, w, bias, out, rows, N, R, coef, sign, per_head);
+    lowrank_up_kernel<float><<<grid, threads, 0, stream>>>(static_cast<const float*>(mid), ldm, w, bias, out, rows, N, R, coef, sign, per_head, mid_tanh, double_exp);
   else if (dtype == kBF16)
-    lowrank_up_kernel<bf16_t><<<grid, threads, 0, stream>>>(static_cast<const bf16_t*>(mid), ldm, w, bias, out, rows, N, R, coef, sign, per_head);
+    lowrank_up_kernel<bf16_t><<<grid, threads, 0, stream>>>(static_cast<const bf16_t*>(mid), ldm, w, bias, out, rows, N, R, coef, sign, per_head, mid_tanh, double_exp);
   else
     LYP_REQUIRE(false, "lowrank_up: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("lowrank_up");

@@ -29,7 +29,8 @@ __device__ __forceinline__ int owner_of(const int32_t* __restrict__ q_start, int
 
 // ------------------------------------------------------ a normed branch joins
 // h[row] += mult * y[row] / rms(y[row]) * wb (+ shift); optionally the row is
-// then normed with w_next into out.  With `rows` the r-th output row is row
+// then normed with w_next into out (out without w_next: the joined row as it is, for a
+// consumer that reads the stream itself).  With `rows` the r-th output row is row
 // rows[r] and h is left alone (the last norm before the output head).
 // y == nullptr: nothing joins (only shift and the following norm).
 template <typename TY, typename T>
@@ -64,10 +65,14 @@ __global__ void branch_join_kernel(float* __restrict__ h, const TY* __restrict__
     if (!rows) hrow[i] = v;
     ss += v * v;
   }
-  if (!w_next) return;
+  if (!out) return;
+  T* orow = out + static_cast<size_t>(r) * H;
+  if (!w_next) {   // no norm follows: the joined row itself, in the activations' type
+    for (int i = threadIdx.x; i < H; i += blockDim.x) orow[i] = from_f32<T>(rows ? joined(i) : hrow[i]);
+    return;
+  }
   ss = block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / static_cast<float>(H) + eps_next);
-  T* orow = out + static_cast<size_t>(r) * H;
   for (int i = threadIdx.x; i < H; i += blockDim.x) {
     const float v = rows ? joined(i) : hrow[i];   // a thread reads back what it wrote itself
     orow[i] = from_f32<T>((v * inv) * w_next[i]);
@@ -140,10 +145,23 @@ __global__ void branch_join_vec_kernel(float* __restrict__ h, const TY* __restri
       for (int i = 0; i < 4; ++i) ss += hv[v][i] * hv[v][i];
     }
   }
-  if (!w_next) return;
+  if (!out) return;
+  Vec4T* orow = reinterpret_cast<Vec4T*>(out + static_cast<size_t>(r) * H);
+  if (!w_next) {   // no norm follows: the joined row itself, in the activations' type
+#pragma unroll
+    for (int v = 0; v < MAXV; ++v) {
+      const int idx = threadIdx.x + v * blockDim.x;
+      if (idx < nvec) {
+        Vec4T o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = from_f32<T>(hv[v][i]);
+        orow[idx] = o;
+      }
+    }
+    return;
+  }
   ss = block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / static_cast<float>(H) + eps_next);
-  Vec4T* orow = reinterpret_cast<Vec4T*>(out + static_cast<size_t>(r) * H);
   const int hist = taps - 1;
   bool fresh = true;
   T* st = nullptr;
@@ -199,7 +217,7 @@ template <typename T>
 __global__ void short_conv_kernel(const T* __restrict__ x, const float* __restrict__ w, T* __restrict__ state,
                                   const int32_t* __restrict__ q_start, const int32_t* __restrict__ positions,
                                   const int32_t* __restrict__ slots, T* __restrict__ out, int n_rows, int B, int C,
-                                  int taps, int residual, int ldx, int act) {
+                                  int taps, int residual, int ldx, int act, const float* __restrict__ bias) {
   const int c = blockIdx.y * blockDim.x + threadIdx.x;
   const int item = blockIdx.x;
   const int hist = taps - 1;
@@ -213,7 +231,7 @@ __global__ void short_conv_kernel(const T* __restrict__ x, const float* __restri
     }
     if (i < hist) return;
     const float* wc = w + static_cast<size_t>(c) * taps;
-    float acc = residual ? to_f32(x[static_cast<size_t>(item) * ldx + c]) : 0.f;
+    float acc = (residual ? to_f32(x[static_cast<size_t>(item) * ldx + c]) : 0.f) + (bias ? bias[c] : 0.f);
     for (int j = 0; j < taps; ++j) acc += wc[j] * to_f32(x[static_cast<size_t>(item - hist + j) * ldx + c]);
     out[static_cast<size_t>(item) * C + c] = from_f32<T>(act ? conv_silu(acc) : acc);
     return;
@@ -232,7 +250,7 @@ __global__ void short_conv_kernel(const T* __restrict__ x, const float* __restri
   const float* wc = w + static_cast<size_t>(c) * taps;
   const int head = n < hist ? n : hist;
   for (int i = 0; i < head; ++i) {
-    float acc = residual ? input(i) : 0.f;
+    float acc = (residual ? input(i) : 0.f) + (bias ? bias[c] : 0.f);
     for (int j = 0; j < taps; ++j) acc += wc[j] * input(i - hist + j);
     out[static_cast<size_t>(q0 + i) * C + c] = from_f32<T>(act ? conv_silu(acc) : acc);
   }
@@ -251,7 +269,7 @@ template <typename T>
 __global__ void short_conv_vec_kernel(const T* __restrict__ x, const float* __restrict__ w, T* __restrict__ state,
                                       const int32_t* __restrict__ q_start, const int32_t* __restrict__ positions,
                                       const int32_t* __restrict__ slots, T* __restrict__ out, int n_rows, int B, int C,
-                                      int taps, int residual, int ldx, int act) {
+                                      int taps, int residual, int ldx, int act, const float* __restrict__ bias) {
   constexpr int VEC = 16 / sizeof(T);
   typedef T VecT __attribute__((ext_vector_type(VEC)));
   const int c = (blockIdx.y * blockDim.x + threadIdx.x) * VEC;
@@ -271,6 +289,9 @@ __global__ void short_conv_vec_kernel(const T* __restrict__ x, const float* __re
   for (int e = 0; e < VEC; ++e)
 #pragma unroll
     for (int j = 0; j < kConvTaps; ++j) wr[e][j] = j < taps ? w[static_cast<size_t>(c + e) * taps + j] : 0.f;
+  float br[VEC];
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) br[e] = bias ? bias[c + e] : 0.f;
   if (item < groups) {
     const int live = q_start[B];
     for (int row = item * kConvRows; row < min(n_rows, (item + 1) * kConvRows); ++row) {
@@ -284,7 +305,7 @@ __global__ void short_conv_vec_kernel(const T* __restrict__ x, const float* __re
       const int b = owner_of(q_start, B, row);
       if (row - q_start[b] < hist) continue;   // the request's item does the rows that read its slot
 #pragma unroll
-      for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+      for (int e = 0; e < VEC; ++e) acc[e] = br[e];
 #pragma unroll
       for (int j = 0; j < kConvTaps; ++j) {
         if (j < taps) {
@@ -316,7 +337,7 @@ __global__ void short_conv_vec_kernel(const T* __restrict__ x, const float* __re
   for (int i = 0; i < head; ++i) {
     float acc[VEC];
 #pragma unroll
-    for (int e = 0; e < VEC; ++e) acc[e] = 0.f;
+    for (int e = 0; e < VEC; ++e) acc[e] = br[e];
 #pragma unroll
     for (int j = 0; j < kConvTaps; ++j) {
       if (j < taps) {
@@ -680,12 +701,13 @@ int lyp_branch_join(float* h, const void* y, int y_dtype, const float* wb, float
   LYP_REQUIRE(n_rows >= 0 && H > 0, "branch_join: bad sizes rows=%d H=%d", n_rows, H);
   LYP_REQUIRE(y == nullptr || wb != nullptr, "branch_join: a branch without its norm's weights");
   LYP_REQUIRE(w_next == nullptr || out != nullptr, "branch_join: a following norm without an output");
-  LYP_REQUIRE(rows == nullptr || w_next != nullptr, "branch_join: selected rows are only normed");
+  LYP_REQUIRE(rows == nullptr || out != nullptr, "branch_join: selected rows go to an output");
   if (n_rows == 0) return 0;
   auto aligned = [](const void* p) { return reinterpret_cast<uintptr_t>(p) % 16 == 0; };
   const bool vec = H % 4 == 0 && H <= 16384 && aligned(h) && aligned(y) && aligned(wb) && aligned(shift) &&
                    aligned(w_next) && aligned(out) && aligned(state);
   const bool conv = conv_w != nullptr;
+  if (out == nullptr) act_dtype = kF32;   // nothing is written: any instantiation will do
   LYP_REQUIRE(!conv || (vec && rows == nullptr && w_next != nullptr && taps >= 1 && slots != nullptr &&
                         positions != nullptr && (taps == 1 || state != nullptr)),
               "branch_join: the convolution follows only rows of up to 16384 values in steps of 4 that are all normed");
@@ -726,10 +748,11 @@ int lyp_add_row(float* h, const float* v, int n_rows, int H, hipStream_t stream)
   return 0;
 }
 
-// x [n_rows, >= C] (rows ldx apart), out [n_rows, C] and state [slots, taps - 1, C] of dtype; w float [C, taps].
+// x [n_rows, >= C] (rows ldx apart), out [n_rows, C] and state [slots, taps - 1, C] of dtype; w float [C, taps];
+// bias float [C] or null, added before the activation.
 int lyp_short_conv(const void* x, const float* w, void* state, const int32_t* q_start, const int32_t* positions,
                    const int32_t* slots, void* out, int dtype, int n_rows, int B, int C, int taps, int residual,
-                   int ldx, int act, hipStream_t stream) {
+                   int ldx, int act, const float* bias, hipStream_t stream) {
   LYP_REQUIRE(n_rows >= 0 && B > 0 && C > 0 && taps >= 1, "short_conv: bad sizes rows=%d B=%d C=%d taps=%d", n_rows, B,
               C, taps);
   LYP_REQUIRE(taps == 1 || state != nullptr, "short_conv: %d taps need a state", taps);
@@ -746,11 +769,11 @@ int lyp_short_conv(const void* x, const float* w, void* state, const int32_t* q_
     if (dtype == kF32)
       short_conv_vec_kernel<float><<<vgrid, vt, 0, stream>>>(static_cast<const float*>(x), w,
                                                              static_cast<float*>(state), q_start, positions, slots,
-                                                             static_cast<float*>(out), n_rows, B, C, taps, residual, ldx, act);
+                                                             static_cast<float*>(out), n_rows, B, C, taps, residual, ldx, act, bias);
     else
       short_conv_vec_kernel<bf16_t><<<vgrid, vt, 0, stream>>>(static_cast<const bf16_t*>(x), w,
                                                               static_cast<bf16_t*>(state), q_start, positions, slots,
-                                                              static_cast<bf16_t*>(out), n_rows, B, C, taps, residual, ldx, act);
+                                                              static_cast<bf16_t*>(out), n_rows, B, C, taps, residual, ldx, act, bias);
     LYP_LAUNCH_CHECK("short_conv");
     return 0;
   }
@@ -759,11 +782,11 @@ int lyp_short_conv(const void* x, const float* w, void* state, const int32_t* q_
   if (dtype == kF32)
     short_conv_kernel<float><<<grid, threads, 0, stream>>>(static_cast<const float*>(x), w, static_cast<float*>(state),
                                                            q_start, positions, slots, static_cast<float*>(out), n_rows,
-                                                           B, C, taps, residual, ldx, act);
+                                                           B, C, taps, residual, ldx, act, bias);
   else if (dtype == kBF16)
     short_conv_kernel<bf16_t><<<grid, threads, 0, stream>>>(static_cast<const bf16_t*>(x), w,
                                                             static_cast<bf16_t*>(state), q_start, positions, slots,
-                                                            static_cast<bf16_t*>(out), n_rows, B, C, taps, residual, ldx, act);
+                                                            static_cast<bf16_t*>(out), n_rows, B, C, taps, residual, ldx, act, bias);
   else
     LYP_REQUIRE(false, "short_conv: unknown dtype %d", dtype);
   LYP_LAUNCH_CHECK("short_conv");

@@ -12,7 +12,8 @@
 //     for any key and value size (the matrix-core kernels take equal sizes in
 //     multiples of 16).  A row at position p sees key j when j <= p and
 //     (window == 0 or p - j < window or j < keep_first); the softmax's
-//     denominator also holds exp(sink[head]) when there is a sink.
+//     denominator also holds exp(sink[head]) when there is a sink.  Scores may be capped
+//     (cap * tanh(s / cap)) and lose slopes[head] * (p - j), a penalty on distance.
 //   * stream_add: h += a (+ b) on the 32-bit residual stream.
 //
 // Norms, angles, scores, weights and sums are 32-bit; only loads and stores see
@@ -204,7 +205,7 @@ __global__ __launch_bounds__(kRowsBlock) void attn_rows_kernel(
     const int32_t* __restrict__ block_tables, int table_width, int bs, const int32_t* __restrict__ q_start,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ ctx_len, int B,
     const float* __restrict__ sink, float scale, int window, int keep_first, T* __restrict__ out, int out_stride,
-    int H, int G, int D, int V) {
+    int H, int G, int D, int V, float cap, const float* __restrict__ slopes) {
   extern __shared__ float smem[];
   float* qs = smem;              // D
   float* ps = smem + D;          // kRowsBlock
@@ -241,6 +242,8 @@ __global__ __launch_bounds__(kRowsBlock) void attn_rows_kernel(
         float dot = 0.f;
         for (int i = 0; i < D; ++i) dot += qs[i] * to_f32(krow[i]);
         s = dot * scale;
+        if (cap > 0.f) s = cap * tanhf(s / cap);
+        if (slopes != nullptr) s -= slopes[h] * static_cast<float>(pos - j);
       }
     }
     const float m_new = fmaxf(m, block_max(s, scratch));
@@ -330,7 +333,8 @@ int lyp_qk_norm_rope_kv(void* qkv, int ld, int dtype, const float* wq, const flo
 int lyp_attn_rows(const void* q, int q_stride, const void* kpool, const void* vpool, const int32_t* block_tables,
                   int table_width, int bs, const int32_t* q_start, const int32_t* positions, const int32_t* ctx_len,
                   int B, const float* sink, float scale, int window, int keep_first, void* out, int out_stride,
-                  int dtype, int n_rows, int H, int G, int D, int V, hipStream_t stream) {
+                  int dtype, int n_rows, int H, int G, int D, int V, float cap, const float* slopes,
+                  hipStream_t stream) {
   LYP_REQUIRE(n_rows >= 0 && B > 0 && H > 0 && G > 0 && H % G == 0 && D > 0 && V > 0 && bs > 0 && table_width > 0,
               "attn_rows: bad sizes");
   LYP_REQUIRE(V <= kRowsCols * kRowsBlock, "attn_rows: values of up to %d, not %d", kRowsCols * kRowsBlock, V);
@@ -344,7 +348,7 @@ int lyp_attn_rows(const void* q, int q_stride, const void* kpool, const void* vp
   attn_rows_kernel<T><<<grid, kRowsBlock, lds, stream>>>(                                                       \
       static_cast<const T*>(q), q_stride, static_cast<const T*>(kpool), static_cast<const T*>(vpool),           \
       block_tables, table_width, bs, q_start, positions, ctx_len, B, sink, scale, window, keep_first,           \
-      static_cast<T*>(out), out_stride, H, G, D, V)
+      static_cast<T*>(out), out_stride, H, G, D, V, cap, slopes)
   if (dtype == kF32) LYP_ROWS(float);
   else if (dtype == kBF16) LYP_ROWS(bf16_t);
   else LYP_REQUIRE(false, "attn_rows: unknown dtype %d", dtype);

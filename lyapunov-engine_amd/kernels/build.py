@@ -38,7 +38,7 @@ CXX_FLAGS = ["-O2", "-std=c++20", "-fPIC", "-Wall", "-Wextra"]
 
 CORE_SOURCES = ["kernels/errors.hip", "kernels/elementwise.hip", "kernels/sequence.hip", "kernels/gemm.hip",
                 "kernels/sampler.hip", "kernels/window_attention.hip", "kernels/moe.hip", "kernels/gated_rows.hip",
-                "kernels/linear_scan.hip"]
+                "kernels/linear_scan.hip", "kernels/qkv_prepare.hip", "kernels/recurrent_rows.hip"]
 ATTN_SOURCES = ["kernels/errors.hip", "kernels/attention.hip"]
 LATENT_SOURCES = ["kernels/errors.hip", "kernels/latent_attention.hip"]
 BLAS_SOURCES = ["kernels/errors.hip", "kernels/library_gemm.hip"]   # host code around the vendor's GEMM library

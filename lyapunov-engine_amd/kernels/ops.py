@@ -93,7 +93,7 @@ def core() -> ctypes.CDLL:
                                         c_void_p, c_int, c_void_p]
         lib.lyp_add_row.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p]
         lib.lyp_short_conv.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-                                       c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]
+                                       c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]
         lib.lyp_activation.argtypes = [c_void_p, c_void_p, c_int, c_longlong, c_int, c_void_p, c_void_p]
         lib.lyp_mingru_scan.argtypes = [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                         c_int, c_int, c_int, c_void_p]
@@ -111,7 +111,7 @@ def core() -> ctypes.CDLL:
                                             c_void_p]
         lib.lyp_attn_rows.argtypes = [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p,
                                       c_void_p, c_int, c_void_p, c_float, c_int, c_int, c_void_p, c_int, c_int, c_int,
-                                      c_int, c_int, c_int, c_int, c_void_p]
+                                      c_int, c_int, c_int, c_int, c_float, c_void_p, c_void_p]
         lib.lyp_stream_add.argtypes = [c_void_p, c_void_p, c_int, c_int, c_void_p, c_longlong, c_void_p]
         lib.lyp_moe_route.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]
         lib.lyp_moe_route_splits.argtypes = [c_int, c_int]
@@ -134,7 +134,7 @@ def core() -> ctypes.CDLL:
                                           c_void_p, c_int, c_int, c_int, c_float, c_void_p]
         lib.lyp_add_sinusoid.argtypes = [c_void_p, c_void_p, c_int, c_int, c_double, c_void_p]
         lib.lyp_glu_act.argtypes = [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]
-        lib.lyp_gate_mul.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]
+        lib.lyp_gate_mul.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]
         lib.lyp_weighted_sum.argtypes = [c_void_p, c_int, c_void_p, c_float, c_void_p, c_int, c_float, c_void_p, c_int,
                                          c_int, c_void_p]
         lib.lyp_qkv_bias_temper_kv.argtypes = [c_void_p, c_int, c_void_p, c_void_p, c_float, c_int, c_void_p, c_void_p,
@@ -144,11 +144,20 @@ def core() -> ctypes.CDLL:
         lib.lyp_linear_scan.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, c_int, c_void_p, c_int,
                                         c_void_p, c_void_p, c_float, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
-                                        c_float, c_void_p]
+                                        c_float, c_void_p, c_int, c_int, c_void_p]
         lib.lyp_head_norm_gate.argtypes = [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int, c_int, c_int,
-                                           c_int, c_float, c_int, c_void_p]
+                                           c_int, c_float, c_int, c_int, c_void_p]
         lib.lyp_lowrank_up.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                       c_void_p, c_float, c_int, c_void_p]
+                                       c_void_p, c_float, c_int, c_int, c_int, c_void_p]
+        lib.lyp_qkv_prepare.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p,
+                                        c_int, c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]
+        lib.lyp_shift_mix.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_int, c_int, c_int, c_int, c_void_p]
+        lib.lyp_skip_gate_group_norm.argtypes = [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                                 c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]
+        lib.lyp_gather_gelu_mul.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_int,
+                                            c_int, c_int, c_void_p]
         lib.lyp_moe_choose_grouped.argtypes = [c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                                c_void_p, c_void_p, c_void_p]
         lib.lyp_moe_route_grouped.argtypes = [c_void_p, c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
@@ -903,7 +912,8 @@ def branch_join(h: torch.Tensor, y: torch.Tensor | None, branch_weight: torch.Te
                 conv: tuple | None = None):
     """h += mult * rmsnorm(y) * branch_weight (+ shift, a vector added to every row), in 32-bit on the
     residual stream; with ``next_weight`` the sum's RMS norm times that weight goes to ``out``
-    (activations).  ``rows`` picks the rows to join and norm into ``out`` and leaves h alone.
+    (activations); ``out`` without ``next_weight`` receives the joined rows themselves in its type (for
+    a consumer that reads the stream as it is).  ``rows`` picks the rows to join and norm into ``out`` and leaves h alone.
     y [T, H] in the activations' type or float; None: only shift and norm.
     ``conv`` = (w, state, slots, positions), as ``short_conv`` takes them, for a step in which every
     row is a request of its own that brings one token: the normed rows then pass the short
@@ -928,10 +938,10 @@ def branch_join(h: torch.Tensor, y: torch.Tensor | None, branch_weight: torch.Te
         raise KernelError(f"branch_join: h {tuple(h.shape)} {h.dtype}, y {None if y is None else tuple(y.shape)}")
     if (shift is not None and shift.numel() != H) or (next_weight is not None and next_weight.numel() != H):
         raise KernelError("branch_join: shift and the following norm's weights have one value per feature")
-    if next_weight is not None and (out is None or tuple(out.shape) != (n, H)):
+    if (next_weight is not None and out is None) or (out is not None and tuple(out.shape) != (n, H)):
         raise KernelError("branch_join: the following norm needs an output of one row per joined row")
-    if rows is not None and (rows.dtype != torch.int32 or next_weight is None):
-        raise KernelError("branch_join: rows are int32 and only picked for a following norm")
+    if rows is not None and (rows.dtype != torch.int32 or out is None):
+        raise KernelError("branch_join: rows are int32 and only picked for an output")
     lib = core()
     _check(lib.lyp_branch_join(_p(h), _p(y), _code(y.dtype) if y is not None else 0, _p(branch_weight), float(mult),
                                _p(shift), _p(next_weight), _p(out), _code(out.dtype) if out is not None else 0,
@@ -965,14 +975,17 @@ def _rows_view(t: torch.Tensor, what: str) -> None:
 
 def short_conv(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor | None, q_start: torch.Tensor,
                positions: torch.Tensor, slots: torch.Tensor, out: torch.Tensor, B: int, residual: bool = True,
-               silu: bool = False):
+               silu: bool = False, bias: torch.Tensor | None = None):
     """out = (x +) the causal filter of x over time, channel by channel, request by request:
     w float [C, taps]; ``state`` [slots, taps - 1, C] of x's type holds every request's last inputs
     from earlier steps (not read for a request at position 0) and is brought up to date.  x may be a
-    column range of a wider tensor; ``silu``: the result passes x * sigmoid(x)."""
+    column range of a wider tensor; ``bias`` (float [C]) is added to the filter's sum; ``silu``: the
+    result passes x * sigmoid(x)."""
     _rows_view(x, "short_conv")
-    _dev(w, state, q_start, positions, slots, out)
-    _f32(w)
+    _dev(w, state, q_start, positions, slots, out, bias)
+    _f32(w, bias)
+    if bias is not None and bias.numel() != x.shape[1]:
+        raise KernelError(f"short_conv: a bias of {bias.numel()} values for {x.shape[1]} channels")
     T, C = x.shape
     taps = w.shape[1]
     if tuple(w.shape) != (C, taps) or out.shape != x.shape or out.dtype != x.dtype or out.data_ptr() == x.data_ptr():
@@ -983,7 +996,7 @@ def short_conv(x: torch.Tensor, w: torch.Tensor, state: torch.Tensor | None, q_s
         raise KernelError("short_conv: the step's tables do not fit its rows and requests")
     lib = core()
     _check(lib.lyp_short_conv(_p(x), _p(w), _p(state), _p(q_start), _p(positions), _p(slots), _p(out), _code(x.dtype),
-                              T, B, C, taps, int(residual), x.stride(0), int(silu), _stream()), lib)
+                              T, B, C, taps, int(residual), x.stride(0), int(silu), _p(bias), _stream()), lib)
     return out
 
 
@@ -1332,11 +1345,14 @@ def qk_norm_rope_kv(qkv: torch.Tensor, q_norm: torch.Tensor | None, k_norm: torc
 def attn_rows(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, block_tables: torch.Tensor,
               q_start: torch.Tensor, positions: torch.Tensor, ctx_len: torch.Tensor, *, num_heads: int,
               num_kv_heads: int, dim: int, vdim: int, scale: float, window: int = 0, keep_first: int = 0,
-              sink: torch.Tensor | None = None) -> torch.Tensor:
+              sink: torch.Tensor | None = None, cap: float = 0.0, slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of every row of the step over its request's pages for any key and value size: q a
     view [T, >= H dim], out [T, H vdim].  A row at position p sees key j <= p when window == 0,
-    p - j < window or j < keep_first."""
+    p - j < window or j < keep_first.  ``cap`` > 0: scores become cap * tanh(score / cap);
+    ``slopes`` (float [H]): key j's score loses slopes[head] * (p - j)."""
     _sink_check(sink, num_heads)
+    _sink_check(slopes, num_heads)
+    _dev(slopes)
     _dev(out, kpool, vpool, block_tables, q_start, positions, ctx_len)
     n_pages, bs = kpool.shape[0], kpool.shape[2]
     T = q.shape[0]
@@ -1350,7 +1366,7 @@ def attn_rows(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: to
     _check(lib.lyp_attn_rows(_p(q), q.stride(0), _p(kpool), _p(vpool), _p(block_tables), block_tables.shape[1], bs,
                              _p(q_start), _p(positions), _p(ctx_len), q_start.numel() - 1, _p(sink), float(scale),
                              int(window), int(keep_first), _p(out), out.stride(0), _code(q.dtype), T, num_heads,
-                             num_kv_heads, dim, vdim, _stream()), lib)
+                             num_kv_heads, dim, vdim, float(cap), _p(slopes), _stream()), lib)
     return out
 
 
@@ -1618,16 +1634,18 @@ def glu_act(gate_up: torch.Tensor, activation: str) -> torch.Tensor:
 GATES = {"sigmoid": 0, "silu": 1}
 
 
-def gate_mul(x: torch.Tensor, gate: torch.Tensor, kind: str) -> torch.Tensor:
-    """x *= sigmoid(gate) or silu(gate), in place: x [T, N] activations, gate [T, N] float or of x's
-    type, possibly a column range of a wider tensor."""
+def gate_mul(x: torch.Tensor, gate: torch.Tensor, kind: str, per: int = 1) -> torch.Tensor:
+    """x *= sigmoid(gate) or silu(gate), in place: x [T, N] activations, gate [T, N / per] float or of
+    x's type, possibly a column range of a wider tensor; one gate value serves ``per`` neighbouring
+    values of x (a head's)."""
     _dev(x)
     _rows_view(gate, "gate_mul")
-    if kind not in GATES or gate.shape != x.shape or gate.dtype not in (torch.float32, x.dtype):
+    if kind not in GATES or per < 1 or x.dim() != 2 or tuple(gate.shape) != (x.shape[0], x.shape[1] // per) or \
+            x.shape[1] % per or gate.dtype not in (torch.float32, x.dtype):
         raise KernelError(f"gate_mul: {kind!r}, x {tuple(x.shape)} {x.dtype}, gate {tuple(gate.shape)} {gate.dtype}")
     lib = core()
     _check(lib.lyp_gate_mul(_p(x), _code(x.dtype), _p(gate), gate.stride(0), _code(gate.dtype), x.shape[0], x.shape[1],
-                            GATES[kind], _stream()), lib)
+                            GATES[kind], int(per), _stream()), lib)
     return x
 
 
@@ -1679,25 +1697,35 @@ LINEAR_SCAN_MAX_DIM = 512    # key channels a head of ``linear_scan`` may have
 def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor, zbias: torch.Tensor | None,
                 coef: torch.Tensor, sign: float, state: torch.Tensor, q_start: torch.Tensor, positions: torch.Tensor,
                 slots: torch.Tensor, out: torch.Tensor, B: int, *, num_heads: int, num_kv_heads: int, dim: int,
-                vdim: int, beta: torch.Tensor | None = None, unit: bool = False, q_scale: float = 1.0) -> torch.Tensor:
+                vdim: int, beta: torch.Tensor | None = None, unit: bool = False, q_scale: float = 1.0,
+                bonus: torch.Tensor | None = None, z_per_head: bool = False, key_step: bool = False) -> torch.Tensor:
     """The recurrence with a matrix state per head over the step's rows, request by request, in order:
     S <- diag(g) S (+ the delta rule's correction when ``beta`` is given) + k v^T, out = S^T q, with
     g = exp(-coef[head] * softplus(sign * (z + zbias))); sign 0: z holds the decays themselves.  q, k [T, G dim] and v [T, H vdim] are
     activations (column ranges of wider tensors are fine), z float [T, H dim], beta [T, H] activations
     (before its sigmoid), state float [slots, H, vdim, dim] (a head's matrix transposed), out float
-    [T, H vdim].  ``unit``: q and k become unit vectors per head first; q is multiplied by ``q_scale``."""
+    [T, H vdim].  ``unit``: q and k become unit vectors per head first; q is multiplied by ``q_scale``.
+    ``bonus`` (float [H dim]): the output reads the state before the token's decay and write, plus the
+    token's own outer product weighted by the bonus per key channel: out = (S + diag(bonus) k v^T)^T q,
+    then S <- diag(g) S + k v^T.  ``z_per_head``: z is [T, H] (zbias [H]), one decay for all of a
+    head's key channels; with ``key_step`` the softplus inside that decay also multiplies the key
+    (a step size: S <- g S + step k v^T)."""
     for t, what in ((q, "q"), (k, "k"), (v, "v"), (z, "z")) + (((beta, "beta"),) if beta is not None else ()):
         _rows_view(t, f"linear_scan {what}")
-    _dev(zbias, coef, state, q_start, positions, slots, out)
-    _f32(z, zbias, coef, state, out)
+    _dev(zbias, coef, state, q_start, positions, slots, out, bonus)
+    _f32(z, zbias, coef, state, out, bonus)
+    zw = num_heads if z_per_head else num_heads * dim
+    if (bonus is not None and (bonus.numel() != num_heads * dim or beta is not None)) or (key_step and not z_per_head):
+        raise KernelError("linear_scan: a bonus has one value per head and key channel and no delta rule; a step "
+                          "size comes with one decay per head")
     T = out.shape[0]
     H, G = num_heads, num_kv_heads
     if q.dtype != k.dtype or q.dtype != v.dtype or (beta is not None and beta.dtype != q.dtype) or \
             q.shape[0] != T or k.shape[0] != T or v.shape[0] != T or z.shape[0] != T or \
-            q.shape[1] != G * dim or k.shape[1] != G * dim or v.shape[1] != H * vdim or z.shape[1] != H * dim or \
+            q.shape[1] != G * dim or k.shape[1] != G * dim or v.shape[1] != H * vdim or z.shape[1] != zw or \
             (beta is not None and tuple(beta.shape) != (T, H)) or tuple(out.shape) != (T, H * vdim) or \
             tuple(state.shape[1:]) != (H, vdim, dim) or coef.numel() != H or \
-            (zbias is not None and zbias.numel() != H * dim) or q_start.numel() != B + 1 or slots.numel() != B or \
+            (zbias is not None and zbias.numel() != zw) or q_start.numel() != B + 1 or slots.numel() != B or \
             positions.numel() != T:
         raise KernelError(f"linear_scan: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}, z {tuple(z.shape)}, "
                           f"state {tuple(state.shape)}, out {tuple(out.shape)} for {H}/{G} heads of {dim}/{vdim}")
@@ -1706,34 +1734,38 @@ def linear_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tens
                                z.stride(0), _p(zbias), _p(coef), float(sign), _p(beta),
                                beta.stride(0) if beta is not None else 0, _p(state), _p(q_start), _p(positions), _p(slots),
                                _p(out), out.stride(0), T, B, H, G, dim, vdim, int(beta is not None), int(unit),
-                               float(q_scale), _stream()), lib)
+                               float(q_scale), _p(bonus), int(z_per_head), int(key_step), _stream()), lib)
     return out
 
 
 def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, kind: str, eps: float,
                    dtype: torch.dtype, *, num_heads: int, vdim: int) -> torch.Tensor:
     """o float [T, H vdim]: every head divided by its root mean square over vdim, times ``weight``
-    (float [vdim], shared by the heads), times sigmoid or silu of ``gate`` [T, H vdim] (float or of
+    (float [vdim], shared by the heads, or [H vdim], every head its own), times sigmoid or silu of ``gate`` [T, H vdim] (float or of
     ``dtype``, possibly a column range); -> [T, H vdim] of ``dtype``."""
     _dev(o, weight)
     _rows_view(gate, "head_norm_gate")
     _f32(o, weight)
     T = o.shape[0]
-    if kind not in GATES or tuple(o.shape) != (T, num_heads * vdim) or gate.shape != o.shape or weight.numel() != vdim or \
+    if kind not in GATES or tuple(o.shape) != (T, num_heads * vdim) or gate.shape != o.shape or \
+            weight.numel() not in (vdim, num_heads * vdim) or \
             gate.dtype not in (torch.float32, dtype):
         raise KernelError(f"head_norm_gate: o {tuple(o.shape)}, gate {tuple(gate.shape)} {gate.dtype}, {num_heads} heads of {vdim}")
     out = torch.empty((T, num_heads * vdim), dtype=dtype, device=o.device)
     lib = core()
     _check(lib.lyp_head_norm_gate(_p(o), _p(weight), _p(gate), gate.stride(0), _code(gate.dtype), _p(out), _code(dtype), T,
-                                  num_heads, vdim, float(eps), GATES[kind], _stream()), lib)
+                                  num_heads, vdim, float(eps), GATES[kind],
+                                  int(weight.numel() != vdim), _stream()), lib)
     return out
 
 
 def lowrank_up(mid: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
-               decay_coef: torch.Tensor | None = None, decay_sign: float = 1.0) -> torch.Tensor:
+               decay_coef: torch.Tensor | None = None, decay_sign: float = 1.0, mid_tanh: bool = False,
+               double_exp: bool = False) -> torch.Tensor:
     """float [T, N] = mid @ w.T (+ bias) in 32-bit: mid [T, R] activations (a column range is fine), w float [N, R].
     With ``decay_coef`` (float, one value per head of N / len values) the result y becomes the decay
-    exp(-coef[head] * softplus(decay_sign * y)) that ``linear_scan`` takes with sign 0."""
+    exp(-coef[head] * softplus(decay_sign * y)) that ``linear_scan`` takes with sign 0.  ``mid_tanh``:
+    the inner values pass tanh first; ``double_exp``: the result y becomes the decay exp(-exp(y))."""
     _rows_view(mid, "lowrank_up")
     _dev(w, bias, decay_coef)
     _f32(w, bias, decay_coef)
@@ -1747,7 +1779,110 @@ def lowrank_up(mid: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = N
     if N % heads:
         raise KernelError(f"lowrank_up: {N} values do not split over {heads} heads")
     _check(lib.lyp_lowrank_up(_p(mid), mid.stride(0), _code(mid.dtype), _p(w), _p(bias), _p(out), T, N, R, _p(decay_coef),
-                              float(decay_sign), N // heads, _stream()), lib)
+                              float(decay_sign), N // heads, int(mid_tanh), int(double_exp), _stream()), lib)
+    return out
+
+
+def qkv_prepare(pre: torch.Tensor, dtype: torch.dtype, *, num_heads: int, num_kv_heads: int, dim: int, vdim: int,
+                slots: torch.Tensor, kpool: torch.Tensor, vpool: torch.Tensor, page_size: int,
+                bias: torch.Tensor | None = None, norm: str = "none", q_weight: torch.Tensor | None = None,
+                k_weight: torch.Tensor | None = None, eps: float = 0.0, positions: torch.Tensor | None = None,
+                table: torch.Tensor | None = None, pairing: str = "neighbours", values_from_keys: bool = False,
+                blend: torch.Tensor | None = None, other_values: torch.Tensor | None = None,
+                keep_values: bool = False):
+    """From a float projection pre [T, >= (H + G) dim (+ G vdim)] (queries, keys and, unless the values
+    are the keys, values side by side) to queries [T, H dim] of ``dtype`` (returned) and keys and
+    values in the tokens' page slots: bias added; values taken (the biased key projection itself with
+    ``values_from_keys``), blended with ``other_values`` (float [T, G vdim]) by the number in ``blend``
+    (a float on the device: v <- (1 - b) v + b other) and, with ``keep_values``, returned unblended as
+    float [T, G vdim]; queries and keys RMS-normed per head (``norm`` "head"; weights [dim] shared by
+    the heads, or none) or over the whole projection ("whole"; weights over all of it); the first
+    table.shape[1] values of every head turned by the position, pairs (2i, 2i + 1) ("neighbours") or
+    (i, i + half) ("halves").  -> (q, kept values or None)."""
+    _rows_view(pre, "qkv_prepare")
+    _dev(bias, q_weight, k_weight, positions, table, slots, kpool, vpool, blend, other_values)
+    _f32(pre, bias, q_weight, k_weight, table, blend, other_values)
+    T, H, G = pre.shape[0], num_heads, num_kv_heads
+    n = (H + G) * dim + (0 if values_from_keys else G * vdim)
+    modes = {"none": 0, "head": 1, "whole": 2}
+    pairings = {"neighbours": 0, "halves": 1}
+    rot = table.shape[1] if table is not None else 0
+    n_pages = kpool.shape[0]
+    want_w = {0: (0, 0), 1: (dim, dim), 2: (H * dim, G * dim)}.get(modes.get(norm, -1))
+    if norm not in modes or pairing not in pairings or pre.shape[1] < n or (bias is not None and bias.numel() != n) or \
+            slots.numel() != T or slots.dtype != torch.int32 or (values_from_keys and vdim != dim) or \
+            (rot and (positions is None or positions.numel() != T or positions.dtype != torch.int32)) or \
+            any(w is not None and w.numel() != k for w, k in zip((q_weight, k_weight), want_w)) or \
+            (blend is not None and (other_values is None or tuple(other_values.shape) != (T, G * vdim) or
+                                    other_values.stride(1) != 1)) or \
+            tuple(kpool.shape) != (n_pages, G, page_size, dim) or tuple(vpool.shape) != (n_pages, G, vdim, page_size) or \
+            kpool.dtype != dtype or vpool.dtype != dtype:
+        raise KernelError(f"qkv_prepare: pre {tuple(pre.shape)}, pools {tuple(kpool.shape)} / {tuple(vpool.shape)} "
+                          f"{kpool.dtype} for {H}+{G} heads of {dim}/{vdim}, norm {norm!r}, pairing {pairing!r}, dtype {dtype}")
+    q = torch.empty((T, H * dim), dtype=dtype, device=pre.device)
+    kept = torch.empty((T, G * vdim), dtype=torch.float32, device=pre.device) if keep_values else None
+    lib = core()
+    _check(lib.lyp_qkv_prepare(_p(pre), pre.stride(0), _p(bias), modes[norm], _p(q_weight), _p(k_weight), float(eps),
+                               _p(positions), _p(table), rot, pairings[pairing], int(values_from_keys), _p(blend),
+                               _p(other_values), other_values.stride(0) if other_values is not None else 0, _p(kept),
+                               _p(slots), _p(q), _p(kpool), _p(vpool), _code(dtype), T, H, G, dim, vdim, page_size,
+                               _stream()), lib)
+    return q, kept
+
+
+def shift_mix(x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, q_start: torch.Tensor, positions: torch.Tensor,
+              slots: torch.Tensor, B: int) -> torch.Tensor:
+    """[n, T, C] of x's type: for every row of ``mu`` (float [n, C]) the blend x_t + (x_(t-1) - x_t) * mu
+    of each row with the row before it in its request; the row before a step's first is the request's
+    state slot (``state`` [slots, C] of x's type; zeros for a request at position 0), which then takes
+    the request's last row of this step."""
+    _rows_view(x, "shift_mix")
+    _dev(mu, state, q_start, positions, slots)
+    _f32(mu)
+    T, C = x.shape
+    if mu.dim() != 2 or mu.shape[1] != C or state.dtype != x.dtype or tuple(state.shape[1:]) != (C,) or \
+            q_start.numel() != B + 1 or slots.numel() != B or positions.numel() != T:
+        raise KernelError(f"shift_mix: x {tuple(x.shape)}, mu {tuple(mu.shape)}, state {tuple(state.shape)} {state.dtype}")
+    out = torch.empty((mu.shape[0], T, C), dtype=x.dtype, device=x.device)
+    lib = core()
+    _check(lib.lyp_shift_mix(_p(x), x.stride(0), _p(mu), mu.shape[0], _p(state), _p(q_start), _p(positions), _p(slots),
+                             _p(out), _code(x.dtype), T, B, C, _stream()), lib)
+    return out
+
+
+def skip_gate_group_norm(o: torch.Tensor, x: torch.Tensor, skip: torch.Tensor, z: torch.Tensor, weight: torch.Tensor,
+                         groups: int, eps: float, *, vdim: int) -> torch.Tensor:
+    """[T, N] of x's type: y = (o + skip[head] * x) * silu(z), then every one of ``groups`` equal
+    consecutive parts of y over its root mean square, times ``weight``.  o float [T, N]; x and z
+    activations [T, N] (column ranges are fine); skip float [N / vdim]; weight float [N]."""
+    _rows_view(x, "skip_gate_group_norm x")
+    _rows_view(z, "skip_gate_group_norm z")
+    _dev(o, skip, weight)
+    _f32(o, skip, weight)
+    T, N = o.shape
+    if tuple(x.shape) != (T, N) or tuple(z.shape) != (T, N) or x.dtype != z.dtype or N % vdim or skip.numel() != N // vdim or \
+            weight.numel() != N or groups < 1 or N % groups or not o.is_contiguous():
+        raise KernelError(f"skip_gate_group_norm: o {tuple(o.shape)}, x {tuple(x.shape)}, z {tuple(z.shape)}, {groups} groups")
+    out = torch.empty((T, N), dtype=x.dtype, device=x.device)
+    lib = core()
+    _check(lib.lyp_skip_gate_group_norm(_p(o), _p(x), x.stride(0), _p(skip), _p(z), z.stride(0), _p(weight), _p(out),
+                                        _code(x.dtype), T, N, vdim, groups, float(eps), _stream()), lib)
+    return out
+
+
+def gather_gelu_mul(p: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """[T, N] of the table's type: gelu_tanh(p[t]) * table[tokens[t]], with p [T, N] float or of the
+    table's type and table [vocab, N] (a column range of a wider table is fine)."""
+    _rows_view(p, "gather_gelu_mul p")
+    _rows_view(table, "gather_gelu_mul table")
+    _dev(tokens)
+    T, N = p.shape
+    if table.shape[1] != N or tokens.numel() != T or tokens.dtype != torch.int32 or p.dtype not in (torch.float32, table.dtype):
+        raise KernelError(f"gather_gelu_mul: p {tuple(p.shape)} {p.dtype}, table {tuple(table.shape)} {table.dtype}")
+    out = torch.empty((T, N), dtype=table.dtype, device=p.device)
+    lib = core()
+    _check(lib.lyp_gather_gelu_mul(_p(p), p.stride(0), _code(p.dtype), _p(tokens), _p(table), table.stride(0),
+                                   table.shape[0], _p(out), _code(table.dtype), T, N, _stream()), lib)
     return out
 
 

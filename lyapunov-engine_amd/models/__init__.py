@@ -1,5 +1,5 @@
 """Architectures.  Importing the package registers the built-in one."""
-from . import faledra, llama, ronupel, tonilix  # noqa: F401
+from . import faledra, llama, ronupel, tonilix, vobotar  # noqa: F401
 from .decoder import CacheGroupLayout, CacheLayout, DecoderModel, build_model
 
 __all__ = ["CacheGroupLayout", "CacheLayout", "DecoderModel", "build_model"]

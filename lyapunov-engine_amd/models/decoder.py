@@ -96,17 +96,23 @@ class DecoderModel(Part):
         out = []
         for prefix, part in self.named_parts():
             for ws in part.weight_specs():
-                full = tuple(WeightSource(prefix + s.name, tuple(s.shape)) for s in ws.sources)
+                full = tuple(WeightSource(s.name if s.absolute else prefix + s.name, tuple(s.shape), s.absolute, s.columns)
+                             for s in ws.sources)
                 out.append((part, WeightSpec(ws.attr, full, ws.init, ws.interleave)))
         return out
 
     def expected_tensors(self) -> dict:
         """Tensor name in the model file -> (shape, init kind)."""
         out = {}
+        shared = set()
         for _, ws in self.weight_table():
             for s in ws.sources:
-                if s.name in out:
+                if s.name in out and (s.columns is None or s.name not in shared or out[s.name] != (tuple(s.shape), ws.init)):
                     raise ValueError(f"two parts claim the tensor {s.name!r}")
+                if s.columns is not None:   # parts that take column ranges may share a tensor
+                    if not 0 <= s.columns[0] < s.columns[1] <= s.shape[1]:
+                        raise ValueError(f"columns {s.columns} of the tensor {s.name!r} {tuple(s.shape)}")
+                    shared.add(s.name)
                 out[s.name] = (tuple(s.shape), ws.init)
         return out
 

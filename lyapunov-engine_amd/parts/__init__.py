@@ -1,5 +1,5 @@
 """Parts of a decoder layer.  Importing the package registers the built-in ones."""
-from . import (attention, block, embedding, filters, latent_attention, linear_recurrence, mingru, mlp, norm, rope,  # noqa: F401
+from . import (attention, block, embedding, filters, gated_attention, latent_attention, linear_recurrence, mingru, mlp, norm, rope,  # noqa: F401
                routed_experts, side_by_side, tempered_attention, window_attention)
 from .base import (Block, Embedding, FeedForward, InputFilter, StreamShift, Head, FixedStep, GroupView, LayerCache, Logits, Mixer, Norm, PagedSpec, PageTensor,
                    Part, PositionEncoding, SLOT, StateSpec, StepBatch, StepContext, StepPlan, StepPlanner, WeightSource, WeightSpec)

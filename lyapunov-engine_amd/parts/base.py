@@ -33,6 +33,12 @@ import torch
 class WeightSource:
     name: str              # tensor name in the file, relative to the part's prefix
     shape: tuple           # a negative entry -n: the file decides this size (``free_size``); n when values are made up
+    # True: ``name`` is the tensor's whole name, whatever the part's prefix (a table that the parts of
+    # several layers share)
+    absolute: bool = False
+    # (lo, hi): the part takes these columns of the file's tensor (``shape`` is still the whole
+    # tensor's); several parts may then name the same tensor
+    columns: Optional[tuple] = None
 
 
 def free_size(made_up: int) -> int:

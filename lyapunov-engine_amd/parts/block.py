@@ -216,3 +216,67 @@ def normed(norm, consumer, ctx: StepContext, h, delta):
     if isinstance(delta, ops.PendingLinear):
         delta = delta.run()
     return norm.forward(ctx, h, delta)
+
+
+def stream_rows(ctx: StepContext, h, delta):
+    """h += delta, and the stream's rows as a branch reads them when no norm stands in front of it:
+    h itself in a 32-bit step, its copy in the step's type otherwise (a joining branch's kernel
+    writes that copy on its way)."""
+    if isinstance(delta, ops.JoiningBranch):
+        if ctx.dtype == torch.float32:
+            delta.join(h)
+            return h
+        out = torch.empty(h.shape, dtype=ctx.dtype, device=h.device)
+        return ops.branch_join(h, delta.y, delta.weight, delta.mult, delta.eps, shift=delta.shift, out=out)
+    if isinstance(delta, ops.ScaledBranch):
+        delta = delta.join(h)
+    if delta is not None:
+        ops.stream_add(h, delta)
+    return ops.cast(h, ctx.dtype)
+
+
+@BLOCKS.register("normed_branches")
+class NormedBranchesBlock(Block):
+    """Every branch reads the residual stream itself and passes a norm on its way back:
+
+        h += norm1(mixer(h));  h += norm2(ffn(h));  h += side_norm(side(h))
+
+    The feed-forward branch may be absent (``LayerSpec.ffn`` None); the third branch is there when
+    ``LayerSpec.extra`` has "side" (a feed-forward of the registry, one that may look at the step's
+    token ids) and "side_norm" (its norm).  A branch joins in the kernel that prepares the next
+    branch's input (ops.JoiningBranch); the block returns its last branch still to be joined."""
+
+    def __init__(self, spec: LayerSpec):
+        self.names = dict(spec.names)
+        self.norm1 = NORMS.build(spec.norm1)
+        self.mixer = MIXERS.build(spec.mixer)
+        self.ffn = FEED_FORWARDS.build(spec.ffn) if spec.ffn is not None else None
+        self.norm2 = NORMS.build(spec.norm2) if self.ffn is not None else None
+        unknown = set(spec.extra) - {"side", "side_norm"}
+        if unknown or (("side" in spec.extra) != ("side_norm" in spec.extra)):
+            raise ValueError(f"the normed-branches arrangement takes 'side' with 'side_norm', not {sorted(spec.extra)}")
+        self.side = FEED_FORWARDS.build(spec.extra["side"]) if "side" in spec.extra else None
+        self.side_norm = NORMS.build(spec.extra["side_norm"]) if self.side is not None else None
+        for norm in (self.norm1, self.norm2, self.side_norm):
+            if norm is not None and not hasattr(norm, "branch"):
+                raise ValueError(f"a branch's norm must be able to join it to the stream; {type(norm).__name__} cannot")
+
+    def children(self):
+        n = self.names
+        out = {n["norm1"]: self.norm1, n["mixer"]: self.mixer}
+        if self.ffn is not None:
+            out.update({n["norm2"]: self.norm2, n["ffn"]: self.ffn})
+        if self.side is not None:
+            out.update({n["side"]: self.side, n["side_norm"]: self.side_norm})
+        return out
+
+    def forward(self, ctx: StepContext, h, delta, cache: LayerCache):
+        x = stream_rows(ctx, h, delta)
+        branch = self.norm1.branch(self.mixer.forward(ctx, x, cache))
+        if self.ffn is not None:
+            x = stream_rows(ctx, h, branch)
+            branch = self.norm2.branch(self.ffn.forward(ctx, x))
+        if self.side is not None:
+            x = stream_rows(ctx, h, branch)
+            branch = self.side_norm.branch(self.side.forward(ctx, x))
+        return h, branch

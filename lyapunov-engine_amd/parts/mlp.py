@@ -102,3 +102,40 @@ class SwiGLU(FeedForward):
     def forward(self, ctx: StepContext, x):
         act = ops.linear_swiglu(x, self.gate_up_proj, self.interleave)
         return ops.linear(act, self.down_proj, out_dtype=ctx.dtype, may_split=True, pending=True)
+
+
+@FEED_FORWARDS.register("token_gated")
+class TokenGatedProjection(FeedForward):
+    """A small branch that the token itself gates: with e the token's row of a table (``dim``
+    values; the table may be a column range of a wider tensor that several layers share),
+
+        y = W_proj (gelu_tanh(W_gate x) * e)
+
+    ``table``: the tensor's whole name in the files; ``table_width`` its columns, of which this part
+    takes ``dim`` from ``column`` on."""
+
+    def __init__(self, hidden_size: int, dim: int, vocab_size: int, table: str, table_width: Optional[int] = None,
+                 column: int = 0, names: Optional[dict] = None):
+        width = dim if table_width is None else int(table_width)
+        if dim <= 0 or vocab_size <= 0 or not 0 <= column <= width - dim:
+            raise ValueError(f"token-gated branch: {dim} values from column {column} of a table of {width}")
+        self.hidden_size, self.dim, self.vocab_size = int(hidden_size), int(dim), int(vocab_size)
+        self.table_name, self.table_width, self.column = table, width, int(column)
+        n = dict(gate="gate", proj="proj")
+        n.update(names or {})
+        self.names = n
+        self.gate_proj: Optional[torch.Tensor] = None
+        self.out_proj: Optional[torch.Tensor] = None
+        self.table: Optional[torch.Tensor] = None
+
+    def weight_specs(self):
+        n = self.names
+        return [WeightSpec("gate_proj", (WeightSource(n["gate"], (self.dim, self.hidden_size)),)),
+                WeightSpec("out_proj", (WeightSource(n["proj"], (self.hidden_size, self.dim)),)),
+                WeightSpec("table", (WeightSource(self.table_name, (self.vocab_size, self.table_width), absolute=True,
+                                                  columns=(self.column, self.column + self.dim)),))]
+
+    def forward(self, ctx: StepContext, x):
+        p = ops.linear(x, self.gate_proj, out_dtype=torch.float32)
+        g = ops.gather_gelu_mul(p, ctx.token_ids, self.table)
+        return ops.linear(g, self.out_proj, out_dtype=ctx.dtype)

@@ -19,23 +19,28 @@ from .base import Norm, StepContext, WeightSource, WeightSpec
 
 @NORMS.register("rmsnorm")
 class RMSNorm(Norm):
-    def __init__(self, size: int, eps: float, tensor: str = "weight"):
+    def __init__(self, size: int, eps: float, tensor: str = "weight", one_plus: bool = False):
         """``tensor``: what the weight is called after the part's prefix ("" where the prefix is
-        the tensor's whole name)."""
+        the tensor's whole name).  ``one_plus``: the tensor is stored around zero and the norm
+        multiplies by 1 + tensor (the sum is formed once, in 32-bit)."""
         self.size = size
         self.eps = float(eps)
         self.tensor = tensor
+        self.one_plus = bool(one_plus)
         self.weight: Optional[torch.Tensor] = None
         self._weight_f: Optional[torch.Tensor] = None
+        if self.one_plus:
+            self.can_defer = False     # the folded forms take the stored tensor as the multiplier
 
     def weight_specs(self):
-        return [WeightSpec("weight", (WeightSource(self.tensor, (self.size,)),), init="ones")]
+        return [WeightSpec("weight", (WeightSource(self.tensor, (self.size,)),), init="normal" if self.one_plus else "ones")]
 
     @property
     def weight_f(self) -> torch.Tensor:
-        """The weights as float (made on first use; a norm's weights do not change)."""
+        """The multipliers as float (made on first use; a norm's weights do not change)."""
         if self._weight_f is None:
-            self._weight_f = self.weight.float().contiguous()
+            w = self.weight.float()
+            self._weight_f = (1.0 + w if self.one_plus else w).contiguous()
         return self._weight_f
 
     def branch(self, y, mult: float = 1.0) -> "ops.JoiningBranch":
@@ -70,7 +75,7 @@ class RMSNorm(Norm):
                 return pending
         n = h.shape[0] if rows is None else rows.numel()
         out = torch.empty((n, self.size), dtype=ctx.dtype, device=h.device)
-        return ops.rmsnorm(h, self.weight, self.eps, out, delta=delta, rows=rows)
+        return ops.rmsnorm(h, self.weight_f if self.one_plus else self.weight, self.eps, out, delta=delta, rows=rows)
 
 
 @NORMS.register("group_rmsnorm")

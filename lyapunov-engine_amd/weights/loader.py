@@ -103,7 +103,8 @@ def load_weights(model: DecoderModel, source: TensorSource, dtype: torch.dtype, 
                  f"model, or a buffer the architecture declares ignorable); ignored")
     device = torch.device(device)
     for owner, ws in model.weight_table():
-        pieces = [source.get(s.name) for s in ws.sources]
+        pieces = [source.get(s.name) if s.columns is None else source.get(s.name)[:, s.columns[0]:s.columns[1]]
+                  for s in ws.sources]
         kinds = {kept_dtype(p.dtype, dtype) for p in pieces}
         keep = torch.float32 if torch.float32 in kinds else kinds.pop()
         pieces = [p.to(device=device, dtype=keep, non_blocking=False) for p in pieces]
