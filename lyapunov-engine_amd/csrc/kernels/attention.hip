@@ -202,6 +202,33 @@ __device__ __forceinline__ float lane_groups_max(float m) {
   return a;
 }
 
+// What may be done to a score between the product and the softmax, in the base-2 domain in which
+// the softmax works (the score times scale * log2 e): cap2 > 0 bends it to cap2 * tanh(score / cap2)
+// (cap2 = cap * log2 e), slope2 takes slope2 * (pos - key) off it (slope2 = the head's slope * log2 e).
+struct ScoreShape {
+  float cap2 = 0.f;
+  float slope2 = 0.f;
+  __device__ __forceinline__ bool any() const { return cap2 > 0.f || slope2 != 0.f; }
+  __device__ __forceinline__ float of(float s2, int pos, int key) const {
+    if (cap2 > 0.f) {
+      // tanh(y) = 1 - 2 / (e^(2 y) + 1): right at both ends (the exponential's overflow gives 1); near 0,
+      // where that difference loses its digits, the series y - y^3/3 + 2 y^5/15 - 17 y^7/315
+      const float y = s2 / cap2, y2 = y * y;
+      const float e = fast_exp2(y * (2.0f * kLog2e));
+      const float far = 1.0f - 2.0f / (e + 1.0f);
+      const float near = y * (1.0f + y2 * (-0.33333334f + y2 * (0.13333334f - 0.053968254f * y2)));
+      s2 = cap2 * (fabsf(y) < 0.15f ? near : far);
+    }
+    return s2 - slope2 * static_cast<float>(pos - key);
+  }
+};
+__device__ __forceinline__ ScoreShape score_shape(float cap, const float* slopes, int head) {
+  ScoreShape sh;
+  sh.cap2 = cap * kLog2e;
+  sh.slope2 = slopes != nullptr ? slopes[head] * kLog2e : 0.f;
+  return sh;
+}
+
 // Take the scores of NB consecutive 16-key blocks (s[u]: rows = keys
 // kb0 + 16 u + 4 (l / 16) + i, column = l % 16), update the running state,
 // rescale the output accumulator and return the probabilities as the column
@@ -213,19 +240,22 @@ __device__ __forceinline__ float lane_groups_max(float m) {
 template <typename T, bool MASKED, int NB>
 __device__ __forceinline__ void softmax_group(const f32x4 (&s)[NB], Frag<T> (&pf)[NB], float scale_log2, int kb0,
                                               int pos, int window, int keep, int hi, Softmax& st,
-                                              f32x4 (&o)[kSteps], int lane) {
+                                              f32x4 (&o)[kSteps], int lane, ScoreShape shape = ScoreShape()) {
   float sv[NB][4];
   float mx = LYP_NEG_INF;
+  const bool shaped = __builtin_amdgcn_ballot_w64(shape.any()) != 0;
 #pragma unroll
   for (int u = 0; u < NB; ++u)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
+      const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
+      float v = s[u][i] * scale_log2;
+      if (shaped) v = shape.of(v, pos, key);
       if constexpr (MASKED) {
-        const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
         const bool vis = key <= pos && key < hi && (window == 0 || key > pos - window || key < keep);
-        sv[u][i] = vis ? s[u][i] * scale_log2 : LYP_NEG_INF;
+        sv[u][i] = vis ? v : LYP_NEG_INF;
       } else {
-        sv[u][i] = s[u][i] * scale_log2;
+        sv[u][i] = v;
       }
       mx = fmaxf(mx, sv[u][i]);
     }
@@ -294,7 +324,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const void* vpool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int n_tiles, int nh, int nkv,
-    int bs, int window, float scale_log2, int keep, const float* __restrict__ sink) {
+    int bs, int window, float scale_log2, int keep, const float* __restrict__ sink, float cap,
+    const float* __restrict__ slopes) {
   using PT = PrefillTile<T>;
   constexpr int KT = PT::kKeys, NB = KT / 16, VEC = PT::kVec;
   constexpr int QW = (4 / GH) * QB * 16;  // new tokens per workgroup
@@ -329,6 +360,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const bool wave_active = hw < g && q0_w < q_len;
   const int col = lane % 16;
   const int head = kvh * g + (hw < g ? hw : 0);
+  const ScoreShape shape = score_shape(cap, slopes, head);
 
   Frag<T> qf[QB][kSteps];
   f32x4 o[QB][kSteps];
@@ -494,10 +526,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
                         (window == 0 || kt0 > pos0[b] + 15 - window);
       if (full)
         softmax_group<T, false, NB>(sc[b], pf[b], scale_log2, kt0, pos0[b] + col, window, keep, hi_wg, st[b], o[b],
-                                    lane);
+                                    lane, shape);
       else
         softmax_group<T, true, NB>(sc[b], pf[b], scale_log2, kt0, col_valid[b] ? pos0[b] + col : -1, window, keep,
-                                   hi_wg, st[b], o[b], lane);
+                                   hi_wg, st[b], o[b], lane, shape);
     }
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
@@ -594,24 +626,28 @@ struct WideTile {
 template <bool MASKED, int NB>
 __device__ __forceinline__ void softmax_wide(const f32x4 (&s)[NB], bf16x8 (&pw)[NB / 2], float scale_log2, int kb0,
                                              int pos, int window, int keep, int hi, float& m_run, f32x4& lacc,
-                                             f32x4 (&o)[kSteps], int lane) {
+                                             f32x4 (&o)[kSteps], int lane, ScoreShape shape = ScoreShape()) {
   bool vis[NB][4];
   float mx = LYP_NEG_INF;
+  const bool shaped = __builtin_amdgcn_ballot_w64(shape.any()) != 0;
+  float sv[NB][4];   // shaped scores (base-2 domain); not used otherwise
 #pragma unroll
   for (int u = 0; u < NB; ++u)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
+      const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
+      float v = s[u][i];
+      if (shaped) v = sv[u][i] = shape.of(v * scale_log2, pos, key);
       if constexpr (MASKED) {
-        const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
         vis[u][i] = key <= pos && key < hi && (window == 0 || key > pos - window || key < keep);
-        mx = fmaxf(mx, vis[u][i] ? s[u][i] : LYP_NEG_INF);
+        mx = fmaxf(mx, vis[u][i] ? v : LYP_NEG_INF);
       } else {
         vis[u][i] = true;
-        mx = fmaxf(mx, s[u][i]);
+        mx = fmaxf(mx, v);
       }
     }
   mx = lane_groups_max(mx);
-  const float m_new = fmaxf(m_run, mx * scale_log2);  // the scale is positive
+  const float m_new = fmaxf(m_run, shaped ? mx : mx * scale_log2);  // the scale is positive
   if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
     const float alpha = fast_exp2(m_run - (m_new == LYP_NEG_INF ? 0.f : m_new));  // 0 while nothing was seen
     m_run = m_new;
@@ -627,7 +663,7 @@ __device__ __forceinline__ void softmax_wide(const f32x4 (&s)[NB], bf16x8 (&pw)[
   for (int u = 0; u < NB; ++u)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      float p = fast_exp2(__builtin_fmaf(s[u][i], scale_log2, -m_safe));
+      float p = shaped ? fast_exp2(sv[u][i] - m_safe) : fast_exp2(__builtin_fmaf(s[u][i], scale_log2, -m_safe));
       if constexpr (MASKED) p = vis[u][i] ? p : 0.f;
       pw[u / 2][4 * (u % 2) + i] = from_f32<bf16_t>(p);
     }
@@ -656,7 +692,7 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0, int n_tiles, int nh, int nkv,
     int bs, int window, float scale_log2, const float* __restrict__ sink, int paired, float* __restrict__ part_o,
     float* __restrict__ part_ml,
-    int n_parts, int keep) {
+    int n_parts, int keep, float cap, const float* __restrict__ slopes) {
   using T = bf16_t;
   using WT = WideTile;
   using MMA = Mma16Wide<bf16_t>;
@@ -687,6 +723,7 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
   const int hsub = (blockIdx.x % head_groups) * GH;
   const int hw = hsub + wave % GH;
   const int head = kvh * g + (hw < g ? hw : 0);
+  const ScoreShape shape = score_shape(cap, slopes, head);
   const T* kp = static_cast<const T*>(kpool);
   const T* vp = static_cast<const T*>(vpool);
   const size_t page_stride = static_cast<size_t>(nkv) * bs * HD;  // of both pools, in elements
@@ -853,10 +890,10 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
       const bool full = kt0 + KT - 1 <= pos0 && kt0 >= lo_wg && pos0 + 15 <= pos_last_wg &&
                         (window == 0 || kt0 > pos0 + 15 - window);
       if (full)
-        softmax_wide<false, NB>(sc, pw, scale_log2, kt0, pos0 + col, window, keep, hi_wg, m_run, lacc, o, lane);
+        softmax_wide<false, NB>(sc, pw, scale_log2, kt0, pos0 + col, window, keep, hi_wg, m_run, lacc, o, lane, shape);
       else
         softmax_wide<true, NB>(sc, pw, scale_log2, kt0, col_valid ? pos0 + col : -1, window, keep, hi_wg, m_run, lacc,
-                               o, lane);
+                               o, lane, shape);
 #pragma unroll
       for (int w = 0; w < NWIDE; ++w) {
         lacc = MMA::mma(ones, pw[w], lacc);
@@ -1046,7 +1083,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const int32_t* __restrict__ ctx_len, const int32_t* __restrict__ dec_seqs,
     float* __restrict__ part_o, float* __restrict__ part_ml, int max_parts, int most_keys_per_wave, int nh, int nkv,
     int bs, int window, float scale_log2, T* __restrict__ out, int out_stride, int keep,
-    const float* __restrict__ sink) {
+    const float* __restrict__ sink, float cap, const float* __restrict__ slopes) {
   extern __shared__ float s_decode[];
   const int lane = threadIdx.x % kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);  // the same in every lane: keeps what follows scalar
@@ -1083,6 +1120,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   const int col = lane % 16;
   const bool col_valid = h0 + col < g;
   const int head = kvh * g + h0 + (col_valid ? col : 0);
+  const ScoreShape shape = score_shape(cap, slopes, head);
   const size_t token = q_start[seq];
 
   Frag<T> qf[kSteps];
@@ -1164,10 +1202,10 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     }
     Frag<T> pf[kDecodeDepth];
     if (aligned && kb0 >= lo && kb0 + GK <= k_end)
-      softmax_group<T, false, kDecodeDepth>(s, pf, scale_log2, kb0, pos, window, keep, k_end, st, o, lane);
+      softmax_group<T, false, kDecodeDepth>(s, pf, scale_log2, kb0, pos, window, keep, k_end, st, o, lane, shape);
     else
       softmax_group<T, true, kDecodeDepth>(s, pf, scale_log2, kb0, col_valid ? pos : -1, window, keep, k_end, st, o,
-                                           lane);
+                                           lane, shape);
 #pragma unroll
     for (int u = 0; u < kDecodeDepth; ++u)
 #pragma unroll
@@ -1383,7 +1421,7 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
                      const int32_t* q_start, const int32_t* ctx_len, const int32_t* tile_seq,
                      const int32_t* tile_q0, int n_tiles, int nh, int nkv, int bs, int window, float scale,
                      int pair, float* part_o, float* part_ml, int n_parts, int keep_first, const float* sink,
-                     hipStream_t stream) {
+                     float cap, const float* slopes, hipStream_t stream) {
   if (check_common("attn_prefill", nh, nkv, bs, max_blocks, q_stride, out_stride, window)) return -1;
   LYP_REQUIRE(n_tiles >= 0 && keep_first >= 0, "attn_prefill: %d tiles, %d kept first tokens", n_tiles, keep_first);
   const int keep = window > 0 ? keep_first : 0;   // without a window every key is seen anyway
@@ -1404,7 +1442,7 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
     attn_prefill_kernel<T, GH, QB><<<grid, 256, 0, stream>>>(                                               \
         static_cast<const T*>(q), q_stride, static_cast<T*>(out), out_stride, kpool, vpool, block_tables,   \
         max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window, scale_log2, keep,    \
-        sink);                                                                                              \
+        sink, cap, slopes);                                                                                 \
   } while (0)
 #define LYP_PREFILL_T(T)                    \
   do {                                      \
@@ -1423,7 +1461,7 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
   attn_prefill_wide_kernel<GH, NW, KS><<<grid, NW * KS * kWave, 0, stream>>>(                                 \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), out_stride, kpool, vpool,           \
       block_tables, max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window,            \
-      scale_log2, sink, paired, part_o, part_ml, n_parts, keep)
+      scale_log2, sink, paired, part_o, part_ml, n_parts, keep, cap, slopes)
     // Two sets of waves per unit while the launch has at most `kSplitBelow` workgroups per
     // compute unit: its time is then that of the unit with most keys, not of the sum.
 #define LYP_PREFILL_WIDE(GH, NW)                                                                              \
@@ -1472,7 +1510,8 @@ int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, cons
                     const void* vpool, int dtype, const int32_t* block_tables, int max_blocks,
                     const int32_t* q_start, const int32_t* ctx_len, const int32_t* dec_seqs, int n_seqs,
                     float* part_o, float* part_ml, int max_parts, int part_keys, int nh, int nkv, int bs,
-                    int window, float scale, int keep_first, const float* sink, hipStream_t stream) {
+                    int window, float scale, int keep_first, const float* sink, float cap, const float* slopes,
+                    hipStream_t stream) {
   if (check_common("attn_decode", nh, nkv, bs, max_blocks, q_stride, out_stride, window)) return -1;
   LYP_REQUIRE(n_seqs >= 0 && max_parts > 0 && keep_first >= 0, "attn_decode: %d requests, %d partitions, %d kept",
               n_seqs, max_parts, keep_first);
@@ -1495,7 +1534,7 @@ int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, cons
   attn_decode_kernel<T, WHOLE><<<grid, kDecodeWaves * kWave, lds, stream>>>(                            \
       static_cast<const T*>(q), q_stride, kpool, vpool, block_tables, max_blocks, q_start, ctx_len,      \
       dec_seqs, part_o, part_ml, max_parts, keys_per_wave, nh, nkv, bs, window, scale_log2,              \
-      static_cast<T*>(out), out_stride, keep, sink)
+      static_cast<T*>(out), out_stride, keep, sink, cap, slopes)
 #define LYP_DECODE_T(T)                                                                                  \
   do {                                                                                                   \
     if (whole) {                                                                                         \

@@ -175,11 +175,12 @@ def attention_lib(head_dim: int) -> ctypes.CDLL:
             raise KernelError(f"attention library for head size {head_dim} reports {lib.lyp_attn_head_dim()}")
         lib.lyp_attn_prefill.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                          c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                         c_float, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]
+                                         c_float, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_float, c_void_p,
+                                         c_void_p]
         lib.lyp_attn_prefill_plan.argtypes = [c_int, c_int, c_int, c_int, c_int, c_int]
         lib.lyp_attn_decode.argtypes = [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                         c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_int, c_int, c_int,
-                                        c_int, c_int, c_int, c_float, c_int, c_void_p, c_void_p]
+                                        c_int, c_int, c_int, c_float, c_int, c_void_p, c_float, c_void_p, c_void_p]
         lib.lyp_attn_decode_plan.argtypes = [c_int, c_int, c_int, c_int]
         _attn[head_dim] = lib
     return lib
@@ -1245,7 +1246,8 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool:
                  window: int = 0, scale: float | None = None, pair: bool | None = None,
                  split: bool = True, parts: int = 1, part_o: torch.Tensor | None = None,
                  part_ml: torch.Tensor | None = None, keep_first: int = 0,
-                 sink: torch.Tensor | None = None) -> torch.Tensor:
+                 sink: torch.Tensor | None = None, cap: float = 0.0,
+                 slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of the step's new tokens over the paged cache (which already
     holds their own keys).  q is a view [T, >= nh * hd] whose first nh * hd
     columns are the query heads; a tile is 64 new tokens of one request, and
@@ -1260,8 +1262,12 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool:
     heads * parts * 2 elements.  With a window, ``keep_first`` first tokens of a
     request stay visible whatever the distance; ``sink`` (float, one per query
     head) is a score without key or value that stands in the softmax's
-    denominator once."""
+    denominator once.  ``cap`` > 0 bends every score to cap * tanh(score / cap);
+    ``slopes`` (float, one per query head) takes slopes[head] * (position - key)
+    off the score of a key."""
     _sink_check(sink, num_heads)
+    _sink_check(slopes, num_heads)
+    _dev(slopes)
     if not q.is_cuda or q.dim() != 2:
         raise KernelError("attention: q must be a 2-d GPU tensor")
     bs = _attn_check(q, out, kpool, vpool, block_tables, num_heads, num_kv_heads, head_dim)
@@ -1277,7 +1283,7 @@ def attn_prefill(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool:
                                 _p(block_tables), block_tables.shape[1], _p(q_start), _p(ctx_len), _p(tile_seq),
                                 _p(tile_q0), n_tiles, num_heads, num_kv_heads, bs, window, scale,
                                 (1 if pair is None else int(bool(pair))) | (0 if split else 2), _p(part_o),
-                                _p(part_ml), parts, int(keep_first), _p(sink), _stream()), lib)
+                                _p(part_ml), parts, int(keep_first), _p(sink), float(cap), _p(slopes), _stream()), lib)
     return out
 
 
@@ -1285,15 +1291,18 @@ def attn_decode(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: 
                 block_tables: torch.Tensor, q_start: torch.Tensor, ctx_len: torch.Tensor,
                 dec_seqs: torch.Tensor | None, n_seqs: int, part_o: torch.Tensor, part_ml: torch.Tensor,
                 max_parts: int, part_keys: int, *, num_heads: int, num_kv_heads: int, head_dim: int, window: int = 0,
-                scale: float | None = None, keep_first: int = 0, sink: torch.Tensor | None = None) -> torch.Tensor:
+                scale: float | None = None, keep_first: int = 0, sink: torch.Tensor | None = None, cap: float = 0.0,
+                slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Attention of requests that bring one new token each, split over
     partitions of the context and merged.  ``part_keys`` comes from
     ``attn_decode_plan``; the caller guarantees that no request's context
     exceeds ``max_parts * part_keys`` (the contexts live on the device and are
     not read here: keys beyond that many partitions would silently be left
     out).  ``PagedAttention.decode_launch`` derives both from the step's bound.
-    ``keep_first`` and ``sink``: as for ``attn_prefill``."""
+    ``keep_first``, ``sink``, ``cap`` and ``slopes``: as for ``attn_prefill``."""
     _sink_check(sink, num_heads)
+    _sink_check(slopes, num_heads)
+    _dev(slopes)
     if not q.is_cuda or q.dim() != 2:
         raise KernelError("attention: q must be a 2-d GPU tensor")
     bs = _attn_check(q, out, kpool, vpool, block_tables, num_heads, num_kv_heads, head_dim)
@@ -1307,7 +1316,7 @@ def attn_decode(q: torch.Tensor, out: torch.Tensor, kpool: torch.Tensor, vpool: 
     _check(lib.lyp_attn_decode(_p(q), q.stride(0), _p(out), out.stride(0), _p(kpool), _p(vpool), _code(q.dtype),
                                _p(block_tables), block_tables.shape[1], _p(q_start), _p(ctx_len), _p(dec_seqs),
                                n_seqs, _p(part_o), _p(part_ml), max_parts, part_keys, num_heads, num_kv_heads, bs,
-                               window, scale, int(keep_first), _p(sink), _stream()), lib)
+                               window, scale, int(keep_first), _p(sink), float(cap), _p(slopes), _stream()), lib)
     return out
 
 

@@ -78,8 +78,7 @@ class GatedAttention(Mixer):
         n = dict(q="q", k="k", v="v", bias=".b", q_norm="q.norm", k_norm="k.norm", mix="vmix", sink="sink", g="g", o="o")
         n.update(names or {})
         self.names = n
-        self.matrix_cores = self.dim == self.vdim and self.dim % 16 == 0 and self.dim <= 256 and \
-            self.cap == 0 and self.slope_power == 0
+        self.matrix_cores = self.dim == self.vdim and self.dim % 16 == 0 and self.dim <= 256
         self.gate_cols = {"none": 0, "head": self.num_heads, "element": self.num_heads * self.vdim}[gate]
         self.in_proj = self.in_bias = self.o_proj = self.q_norm = self.k_norm = self.mix = self.sink = None
         self.in_bias_f = self.q_norm_f = self.k_norm_f = self.mix_f = self.sink_f = self.slopes_f = None
@@ -159,7 +158,7 @@ class GatedAttention(Mixer):
                           window=self.window, sink=self.sink_f, cap=self.cap, slopes=self.slopes_f)
         else:
             common = dict(num_heads=H, num_kv_heads=G, head_dim=self.dim, window=self.window, scale=self.scale,
-                          sink=self.sink_f)
+                          sink=self.sink_f, cap=self.cap, slopes=self.slopes_f)
             sizes = dict(num_heads=H, num_kv_heads=G, head_dim=self.dim)
             work = ctx.plans[AttentionWork.key]
             pl = prefill_launch(work.meta, ctx.dtype, g.page_size, window=self.window, **sizes)

@@ -164,9 +164,11 @@ TOL = {"float32": dict(rtol=5e-5, atol=5e-5), "bfloat16": dict(rtol=0.0, atol=8e
 TOL_ALONE = {"float32": dict(rtol=5e-5, atol=5e-5), "bfloat16": dict(rtol=0.0, atol=3e-2, median=1e-2)}
 
 
-def compare(trace: Trace, got: dict, want: dict, dtype: str, label="", tol=None):
+def compare(trace: Trace, got: dict, want: dict, dtype: str, label="", tol=None, slack=None):
     """Every row of every step against the reference logits at its (request,
-    position); on failure name the first wrong place, which is where to look."""
+    position); on failure name the first wrong place, which is where to look.
+    ``slack``: request -> per position, a further allowance in logits for that row (for designs
+    in which single rows are far more sensitive to rounding than the rest)."""
     assert set(got) == set(trace.rows), f"{label}: steps with logits {sorted(got)} != expected {sorted(trace.rows)}"
     tol = tol or TOL[dtype]
     rel = []
@@ -177,7 +179,8 @@ def compare(trace: Trace, got: dict, want: dict, dtype: str, label="", tol=None)
             ref = np.asarray(want[rid][pos], dtype=np.float64)
             scale = max(1.0, float(np.abs(ref).max()))
             err = np.abs(got[n][i].astype(np.float64) - ref)
-            bad = err > tol["atol"] * scale + tol["rtol"] * np.abs(ref)
+            more = float(slack[rid][pos]) if slack is not None else 0.0
+            bad = err > tol["atol"] * scale + tol["rtol"] * np.abs(ref) + more
             assert not bad.any(), (f"{label}: first wrong logits at step {n}, request {rid!r}, position {pos}: "
                                    f"max error {err.max():.3e} (scale {scale:.3f}); entries of the step: "
                                    f"{[(e['id'], len(e['tokens'])) for e in trace.steps[n]['entries']]}")
