@@ -171,8 +171,47 @@ TONILIX_SIZES = {
     "1b": (tonilix_shape(2048, 32, 8, 64, 16, 128256, 8192, 32, 4), DESIGN_SIZES["1b"][0]),
     "wide": (tonilix_shape(4096, 32, 8, 128, 8, 128256, 14336, 32, 4), DESIGN_SIZES["wide"][0]),
 }
+
+
+# Vobotar models with layers of a real model's sizes, three kinds in turn: full attention (capped
+# scores, blended values, a gate on every output value), windowed attention whose values are its keys
+# beside a time mix with a matrix per head, and windowed attention with normed projections beside a
+# state-space layer; every layer with the Llama shape's gated feed-forward and a token-gated branch of
+# 128 values.  Beside each stands the Tonilix model of equal width and depth, the closest design
+# (attention beside a recurrence with a matrix per head, state slots beside pages, a blend with the
+# previous row in front of the mixers).
+def vobotar_shape(width, heads, kv_heads, dim, layers, vocab, ff):
+    rec = max(1, width // 64)
+
+    def full():
+        return dict(type="attention", mlp=dict(kind="dense", ff=ff),
+                    mixer=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, softcap=30.0, v_mix=True,
+                               rot=dict(base=1e6, dims=dim)))
+
+    def keys_pair():
+        return dict(type="parallel", mlp=dict(kind="dense", ff=ff),
+                    mixer=dict(left=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, mask=dict(size=1024)),
+                               right=dict(heads=rec, dim=64), left_scale=0.7, right_scale=0.7))
+
+    def space_pair():
+        return dict(type="parallel_2", mlp=dict(kind="dense", ff=ff),
+                    mixer=dict(left=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, mask=dict(size=1024),
+                                         rot=dict(base=1e4, dims=dim // 2)),
+                               right=dict(heads=2 * rec, vdim=64, state=128, groups=1, conv=4, norm_groups=8),
+                               left_scale=0.7, right_scale=0.7))
+
+    kinds = (full, keys_pair, space_pair)
+    return dict(architecture="Vobotar", vocab=vocab, width=width, embedding=dict(scale=1.0), norm=dict(eps=1e-6),
+                token_side=dict(dim=128), layers=[kinds[i % 3]() for i in range(layers)])
+
+
+VOBOTAR_SIZES = {
+    "small": (vobotar_shape(1024, 16, 4, 64, 8, 32000, 4096), TONILIX_SIZES["small"][0]),
+    "1b": (vobotar_shape(2048, 32, 8, 64, 16, 128256, 8192), TONILIX_SIZES["1b"][0]),
+    "wide": (vobotar_shape(4096, 32, 8, 128, 8, 128256, 14336), TONILIX_SIZES["wide"][0]),
+}
 # what stands beside a design's sizes
-BESIDE = {"faledra": "llama", "ronupel": "llama", "tonilix": "faledra"}
+BESIDE = {"faledra": "llama", "ronupel": "llama", "tonilix": "faledra", "vobotar": "tonilix"}
 
 
 class _Vocab:
@@ -189,7 +228,7 @@ def run_design(args):
 
     context, block_size, out = 2304, 16, {}
     design = args.design
-    sizes = {"faledra": DESIGN_SIZES, "ronupel": RONUPEL_SIZES, "tonilix": TONILIX_SIZES}[design]
+    sizes = {"faledra": DESIGN_SIZES, "ronupel": RONUPEL_SIZES, "tonilix": TONILIX_SIZES, "vobotar": VOBOTAR_SIZES}[design]
     beside = BESIDE[design]
     for size in (args.size.split(",") if args.size else sorted(sizes)):
         other, second = sizes[size]
@@ -433,9 +472,10 @@ def main():
                     help="mixed: the continuous batch of BASELINE.json configs[3] instead of the headline")
     ap.add_argument("--skip-points", action="store_true", help="only the headline decode and the prefill")
     ap.add_argument("--skip-check", action="store_true", help="no comparison of bfloat16 logits with a 32-bit run")
-    ap.add_argument("--design", default="llama", choices=["llama", "faledra", "ronupel", "tonilix"],
-                    help="faledra, ronupel, tonilix: that design's prefill and decode speed at a few sizes, each beside "
-                         "the Llama shape (Tonilix: the Faledra model) of equal size, instead of the headline")
+    ap.add_argument("--design", default="llama", choices=["llama", "faledra", "ronupel", "tonilix", "vobotar"],
+                    help="faledra, ronupel, tonilix, vobotar: that design's prefill and decode speed at a few sizes, each "
+                         "beside the Llama shape (Tonilix: the Faledra model; Vobotar: the Tonilix model) of equal size, "
+                         "instead of the headline")
     ap.add_argument("--size", default="", help="with another --design: which sizes, with commas (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
