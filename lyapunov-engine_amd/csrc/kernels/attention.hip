@@ -207,26 +207,53 @@ __device__ __forceinline__ float lane_groups_max(float m) {
 // (cap2 = cap * log2 e), slope2 takes slope2 * (pos - key) off it (slope2 = the head's slope * log2 e).
 struct ScoreShape {
   float cap2 = 0.f;
+  float inv_cap2 = 0.f;
   float slope2 = 0.f;
   __device__ __forceinline__ bool any() const { return cap2 > 0.f || slope2 != 0.f; }
-  __device__ __forceinline__ float of(float s2, int pos, int key) const {
-    if (cap2 > 0.f) {
-      // tanh(y) = 1 - 2 / (e^(2 y) + 1): right at both ends (the exponential's overflow gives 1); near 0,
-      // where that difference loses its digits, the series y - y^3/3 + 2 y^5/15 - 17 y^7/315
-      const float y = s2 / cap2, y2 = y * y;
-      const float e = fast_exp2(y * (2.0f * kLog2e));
-      const float far = 1.0f - 2.0f / (e + 1.0f);
-      const float near = y * (1.0f + y2 * (-0.33333334f + y2 * (0.13333334f - 0.053968254f * y2)));
-      s2 = cap2 * (fabsf(y) < 0.15f ? near : far);
-    }
-    return s2 - slope2 * static_cast<float>(pos - key);
+  // the bent score from the raw product s (scale2 = scale * log2 e): tanh(y) = 1 - 2 / (e^(2 y) + 1), right
+  // at both ends (the exponential's overflow gives 1).  PRECISE: near 0, where that difference loses its
+  // digits (an error of 1e-7 of the cap), the series y - y^3/3 + 2 y^5/15 - 17 y^7/315 instead; operands
+  // that were rounded to 16 bits are a thousand times coarser than that, and take the short form.
+  template <bool PRECISE>
+  __device__ __forceinline__ float capped(float s, float scale2) const {
+    const float y = s * (scale2 * inv_cap2);
+    const float e = fast_exp2(y * (2.0f * kLog2e));
+    const float far = __builtin_fmaf(-2.0f * cap2, __builtin_amdgcn_rcpf(e + 1.0f), cap2);
+    if constexpr (!PRECISE) return far;
+    const float y2 = y * y;
+    const float near = cap2 * y * (1.0f + y2 * (-0.33333334f + y2 * (0.13333334f - 0.053968254f * y2)));
+    return fabsf(y) < 0.15f ? near : far;
   }
 };
 __device__ __forceinline__ ScoreShape score_shape(float cap, const float* slopes, int head) {
   ScoreShape sh;
   sh.cap2 = cap * kLog2e;
+  sh.inv_cap2 = cap > 0.f ? 1.0f / sh.cap2 : 0.f;
   sh.slope2 = slopes != nullptr ? slopes[head] * kLog2e : 0.f;
   return sh;
+}
+// The scores of NB consecutive 16-key blocks, scaled and shaped in place (s[u]: rows = keys
+// kb0 + 16 u + 4 (l / 16) + i, column at position pos); the softmax that follows takes a scale of 1.
+// One branch around each pass over the scores, none inside.
+template <int NB, bool PRECISE>
+__device__ __forceinline__ void shape_scores(f32x4 (&s)[NB], float scale_log2, int kb0, int pos, int lane,
+                                             const ScoreShape& shape) {
+  if (shape.cap2 > 0.f) {
+#pragma unroll
+    for (int u = 0; u < NB; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s[u][i] = shape.template capped<PRECISE>(s[u][i], scale_log2);
+  } else {
+#pragma unroll
+    for (int u = 0; u < NB; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) s[u][i] *= scale_log2;
+  }
+  const float d0 = static_cast<float>(pos - kb0 - 4 * (lane / 16));
+#pragma unroll
+  for (int u = 0; u < NB; ++u)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) s[u][i] -= shape.slope2 * (d0 - static_cast<float>(16 * u + i));
 }
 
 // Take the scores of NB consecutive 16-key blocks (s[u]: rows = keys
@@ -240,22 +267,19 @@ __device__ __forceinline__ ScoreShape score_shape(float cap, const float* slopes
 template <typename T, bool MASKED, int NB>
 __device__ __forceinline__ void softmax_group(const f32x4 (&s)[NB], Frag<T> (&pf)[NB], float scale_log2, int kb0,
                                               int pos, int window, int keep, int hi, Softmax& st,
-                                              f32x4 (&o)[kSteps], int lane, ScoreShape shape = ScoreShape()) {
+                                              f32x4 (&o)[kSteps], int lane) {
   float sv[NB][4];
   float mx = LYP_NEG_INF;
-  const bool shaped = __builtin_amdgcn_ballot_w64(shape.any()) != 0;
 #pragma unroll
   for (int u = 0; u < NB; ++u)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
-      float v = s[u][i] * scale_log2;
-      if (shaped) v = shape.of(v, pos, key);
       if constexpr (MASKED) {
+        const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
         const bool vis = key <= pos && key < hi && (window == 0 || key > pos - window || key < keep);
-        sv[u][i] = vis ? v : LYP_NEG_INF;
+        sv[u][i] = vis ? s[u][i] * scale_log2 : LYP_NEG_INF;
       } else {
-        sv[u][i] = v;
+        sv[u][i] = s[u][i] * scale_log2;
       }
       mx = fmaxf(mx, sv[u][i]);
     }
@@ -361,6 +385,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const int col = lane % 16;
   const int head = kvh * g + (hw < g ? hw : 0);
   const ScoreShape shape = score_shape(cap, slopes, head);
+  const bool shaped = __builtin_amdgcn_ballot_w64(shape.any()) != 0;   // the same in every lane
 
   Frag<T> qf[QB][kSteps];
   f32x4 o[QB][kSteps];
@@ -524,12 +549,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       // every token of the block sees the whole tile: no masks
       const bool full = kt0 + KT - 1 <= pos0[b] && kt0 >= lo_wg && pos0[b] + 15 <= pos_last_wg &&
                         (window == 0 || kt0 > pos0[b] + 15 - window);
+      if (shaped) shape_scores<NB, sizeof(T) == 4>(sc[b], scale_log2, kt0, pos0[b] + col, lane, shape);
+      const float sm_scale = shaped ? 1.0f : scale_log2;
       if (full)
-        softmax_group<T, false, NB>(sc[b], pf[b], scale_log2, kt0, pos0[b] + col, window, keep, hi_wg, st[b], o[b],
-                                    lane, shape);
+        softmax_group<T, false, NB>(sc[b], pf[b], sm_scale, kt0, pos0[b] + col, window, keep, hi_wg, st[b], o[b],
+                                    lane);
       else
-        softmax_group<T, true, NB>(sc[b], pf[b], scale_log2, kt0, col_valid[b] ? pos0[b] + col : -1, window, keep,
-                                   hi_wg, st[b], o[b], lane, shape);
+        softmax_group<T, true, NB>(sc[b], pf[b], sm_scale, kt0, col_valid[b] ? pos0[b] + col : -1, window, keep,
+                                   hi_wg, st[b], o[b], lane);
     }
 #pragma unroll
     for (int u = 0; u < NB; ++u) {
@@ -626,28 +653,24 @@ struct WideTile {
 template <bool MASKED, int NB>
 __device__ __forceinline__ void softmax_wide(const f32x4 (&s)[NB], bf16x8 (&pw)[NB / 2], float scale_log2, int kb0,
                                              int pos, int window, int keep, int hi, float& m_run, f32x4& lacc,
-                                             f32x4 (&o)[kSteps], int lane, ScoreShape shape = ScoreShape()) {
+                                             f32x4 (&o)[kSteps], int lane) {
   bool vis[NB][4];
   float mx = LYP_NEG_INF;
-  const bool shaped = __builtin_amdgcn_ballot_w64(shape.any()) != 0;
-  float sv[NB][4];   // shaped scores (base-2 domain); not used otherwise
 #pragma unroll
   for (int u = 0; u < NB; ++u)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
-      float v = s[u][i];
-      if (shaped) v = sv[u][i] = shape.of(v * scale_log2, pos, key);
       if constexpr (MASKED) {
+        const int key = kb0 + 16 * u + 4 * (lane / 16) + i;
         vis[u][i] = key <= pos && key < hi && (window == 0 || key > pos - window || key < keep);
-        mx = fmaxf(mx, vis[u][i] ? v : LYP_NEG_INF);
+        mx = fmaxf(mx, vis[u][i] ? s[u][i] : LYP_NEG_INF);
       } else {
         vis[u][i] = true;
-        mx = fmaxf(mx, v);
+        mx = fmaxf(mx, s[u][i]);
       }
     }
   mx = lane_groups_max(mx);
-  const float m_new = fmaxf(m_run, shaped ? mx : mx * scale_log2);  // the scale is positive
+  const float m_new = fmaxf(m_run, mx * scale_log2);  // the scale is positive
   if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
     const float alpha = fast_exp2(m_run - (m_new == LYP_NEG_INF ? 0.f : m_new));  // 0 while nothing was seen
     m_run = m_new;
@@ -663,7 +686,7 @@ __device__ __forceinline__ void softmax_wide(const f32x4 (&s)[NB], bf16x8 (&pw)[
   for (int u = 0; u < NB; ++u)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      float p = shaped ? fast_exp2(sv[u][i] - m_safe) : fast_exp2(__builtin_fmaf(s[u][i], scale_log2, -m_safe));
+      float p = fast_exp2(__builtin_fmaf(s[u][i], scale_log2, -m_safe));
       if constexpr (MASKED) p = vis[u][i] ? p : 0.f;
       pw[u / 2][4 * (u % 2) + i] = from_f32<bf16_t>(p);
     }
@@ -684,8 +707,10 @@ struct TileRegs {
 // tiles 1, 3, 5, ..., each through LDS buffers of its own, and the two running results are merged
 // at the end.  Half as many tiles in a row for one unit: for launches with few units, whose time
 // is that of the unit with most keys.
-template <int GH, int NW, int KS>
-__global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_wide_kernel(
+// SHAPED: scores are capped or pay for distance (ScoreShape); an instantiation of its own, with room
+// for the registers that takes, so that the plain form keeps its four workgroups a compute unit.
+template <int GH, int NW, int KS, bool SHAPED>
+__global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? (SHAPED ? 2 : 4) : 1) void attn_prefill_wide_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride, const void* kpool,
     const void* vpool, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ q_start, const int32_t* __restrict__ ctx_len,
@@ -723,7 +748,7 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
   const int hsub = (blockIdx.x % head_groups) * GH;
   const int hw = hsub + wave % GH;
   const int head = kvh * g + (hw < g ? hw : 0);
-  const ScoreShape shape = score_shape(cap, slopes, head);
+  const ScoreShape shape = SHAPED ? score_shape(cap, slopes, head) : ScoreShape();
   const T* kp = static_cast<const T*>(kpool);
   const T* vp = static_cast<const T*>(vpool);
   const size_t page_stride = static_cast<size_t>(nkv) * bs * HD;  // of both pools, in elements
@@ -874,7 +899,7 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
     };
 
     // ---- one tile's worth of work for this wave
-    auto compute = [&](int buf, int kt0) {
+    auto compute = [&](int buf, int kt0) __attribute__((always_inline)) {
       const T* ks = lds + buf * WT::kElems;
       const T* vs = ks + KT * WT::kKLd;
       f32x4 sc[NB];
@@ -889,11 +914,13 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
       bf16x8 pw[NWIDE];
       const bool full = kt0 + KT - 1 <= pos0 && kt0 >= lo_wg && pos0 + 15 <= pos_last_wg &&
                         (window == 0 || kt0 > pos0 + 15 - window);
+      if constexpr (SHAPED) shape_scores<NB, false>(sc, scale_log2, kt0, pos0 + col, lane, shape);
+      const float sm_scale = SHAPED ? 1.0f : scale_log2;
       if (full)
-        softmax_wide<false, NB>(sc, pw, scale_log2, kt0, pos0 + col, window, keep, hi_wg, m_run, lacc, o, lane, shape);
+        softmax_wide<false, NB>(sc, pw, sm_scale, kt0, pos0 + col, window, keep, hi_wg, m_run, lacc, o, lane);
       else
-        softmax_wide<true, NB>(sc, pw, scale_log2, kt0, col_valid ? pos0 + col : -1, window, keep, hi_wg, m_run, lacc,
-                               o, lane, shape);
+        softmax_wide<true, NB>(sc, pw, sm_scale, kt0, col_valid ? pos0 + col : -1, window, keep, hi_wg, m_run, lacc,
+                               o, lane);
 #pragma unroll
       for (int w = 0; w < NWIDE; ++w) {
         lacc = MMA::mma(ones, pw[w], lacc);
@@ -907,7 +934,7 @@ __global__ __launch_bounds__(NW* KS* kWave, HD <= 64 ? 4 : 1) void attn_prefill_
     // One round of the loop, in tiles of this set: tile kt0 is in LDS buffer `buf`, the next in
     // `ready`; the loads of the one after that are started into `filling`, whose last content is
     // in LDS already.  A set whose tile lies past the unit's keys still passes the barriers.
-    auto step = [&](int kt0, int buf, TileRegs<PER>& filling, const TileRegs<PER>& ready) {
+    auto step = [&](int kt0, int buf, TileRegs<PER>& filling, const TileRegs<PER>& ready) __attribute__((always_inline)) {
       int page_n[PER], page_off_n[PER];
       read_table(page_n, page_off_n);      // for the third tile after kt0
       ask(filling, page, page_off);        // the second after kt0
@@ -1121,6 +1148,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   const bool col_valid = h0 + col < g;
   const int head = kvh * g + h0 + (col_valid ? col : 0);
   const ScoreShape shape = score_shape(cap, slopes, head);
+  const bool shaped = __builtin_amdgcn_ballot_w64(shape.any()) != 0;   // the same in every lane
   const size_t token = q_start[seq];
 
   Frag<T> qf[kSteps];
@@ -1201,11 +1229,13 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
       for (int u = 0; u < kDecodeDepth; ++u) load_k_of(u, kb_next + 16 * u);
     }
     Frag<T> pf[kDecodeDepth];
+    if (shaped) shape_scores<kDecodeDepth, sizeof(T) == 4>(s, scale_log2, kb0, pos, lane, shape);
+    const float sm_scale = shaped ? 1.0f : scale_log2;
     if (aligned && kb0 >= lo && kb0 + GK <= k_end)
-      softmax_group<T, false, kDecodeDepth>(s, pf, scale_log2, kb0, pos, window, keep, k_end, st, o, lane, shape);
+      softmax_group<T, false, kDecodeDepth>(s, pf, sm_scale, kb0, pos, window, keep, k_end, st, o, lane);
     else
-      softmax_group<T, true, kDecodeDepth>(s, pf, scale_log2, kb0, col_valid ? pos : -1, window, keep, k_end, st, o,
-                                           lane, shape);
+      softmax_group<T, true, kDecodeDepth>(s, pf, sm_scale, kb0, col_valid ? pos : -1, window, keep, k_end, st, o,
+                                           lane);
 #pragma unroll
     for (int u = 0; u < kDecodeDepth; ++u)
 #pragma unroll
@@ -1457,11 +1487,16 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
     // (0: no); bit 1 forbids the two sets of waves per unit (for tests and measurements).
     // Units (workgroups before pairing) beyond one per compute unit share compute units anyway;
     // pairing then evens out the causal mask's triangle of work.
-#define LYP_PREFILL_WIDE_KS(GH, NW, KS)                                                                       \
-  attn_prefill_wide_kernel<GH, NW, KS><<<grid, NW * KS * kWave, 0, stream>>>(                                 \
+#define LYP_PREFILL_WIDE_KSS(GH, NW, KS, SH)                                                                  \
+  attn_prefill_wide_kernel<GH, NW, KS, SH><<<grid, NW * KS * kWave, 0, stream>>>(                             \
       static_cast<const bf16_t*>(q), q_stride, static_cast<bf16_t*>(out), out_stride, kpool, vpool,           \
       block_tables, max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window,            \
       scale_log2, sink, paired, part_o, part_ml, n_parts, keep, cap, slopes)
+#define LYP_PREFILL_WIDE_KS(GH, NW, KS)                      \
+  do {                                                       \
+    if (cap > 0.f || slopes != nullptr) LYP_PREFILL_WIDE_KSS(GH, NW, KS, true); \
+    else LYP_PREFILL_WIDE_KSS(GH, NW, KS, false);            \
+  } while (0)
     // Two sets of waves per unit while the launch has at most `kSplitBelow` workgroups per
     // compute unit: its time is then that of the unit with most keys, not of the sum.
 #define LYP_PREFILL_WIDE(GH, NW)                                                                              \
@@ -1484,6 +1519,7 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
     else LYP_PREFILL_WIDE(1, 4);
 #undef LYP_PREFILL_WIDE
 #undef LYP_PREFILL_WIDE_KS
+#undef LYP_PREFILL_WIDE_KSS
     if (n_parts > 1)
       attn_merge_parts_kernel<bf16_t><<<dim3(nh, 64, n_tiles), 64, 0, stream>>>(
           part_o, part_ml, n_parts, q_start, tile_seq, tile_q0, static_cast<bf16_t*>(out), out_stride, nh, sink);

@@ -48,7 +48,7 @@ class RMSNorm(Norm):
         if isinstance(y, ops.PendingLinear):
             y = y.run()
         if y.dim() == 3:
-            y = ops.sum_parts(y, torch.float32)
+            y = y[0] if y.shape[0] == 1 else ops.sum_parts(y, torch.float32)     # one slice: nothing to add up
         return ops.JoiningBranch(y, self.weight_f, self.eps, mult)
 
     # A delta may be an ops.JoiningBranch: the sum and this norm are then one kernel.
