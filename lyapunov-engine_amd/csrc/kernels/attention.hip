@@ -342,7 +342,7 @@ struct PrefillTile {
   static constexpr int kPerThread = (kKVecs + 255) / 256;
 };
 
-template <typename T, int GH, int QB>
+template <typename T, int GH, int QB, bool SHAPED>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride, const void* kpool,
     const void* vpool, const int32_t* __restrict__ block_tables, int max_blocks,
@@ -384,8 +384,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
   const bool wave_active = hw < g && q0_w < q_len;
   const int col = lane % 16;
   const int head = kvh * g + (hw < g ? hw : 0);
-  const ScoreShape shape = score_shape(cap, slopes, head);
-  const bool shaped = __builtin_amdgcn_ballot_w64(shape.any()) != 0;   // the same in every lane
+  const ScoreShape shape = SHAPED ? score_shape(cap, slopes, head) : ScoreShape();
 
   Frag<T> qf[QB][kSteps];
   f32x4 o[QB][kSteps];
@@ -549,8 +548,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       // every token of the block sees the whole tile: no masks
       const bool full = kt0 + KT - 1 <= pos0[b] && kt0 >= lo_wg && pos0[b] + 15 <= pos_last_wg &&
                         (window == 0 || kt0 > pos0[b] + 15 - window);
-      if (shaped) shape_scores<NB, sizeof(T) == 4>(sc[b], scale_log2, kt0, pos0[b] + col, lane, shape);
-      const float sm_scale = shaped ? 1.0f : scale_log2;
+      if constexpr (SHAPED) shape_scores<NB, sizeof(T) == 4>(sc[b], scale_log2, kt0, pos0[b] + col, lane, shape);
+      const float sm_scale = SHAPED ? 1.0f : scale_log2;
       if (full)
         softmax_group<T, false, NB>(sc[b], pf[b], sm_scale, kt0, pos0[b] + col, window, keep, hi_wg, st[b], o[b],
                                     lane);
@@ -1103,7 +1102,7 @@ constexpr int decode_lds_floats(int g) { return kDecodeWaves * ((g < 16 ? g : 16
 
 // WHOLE: the launch has one partition per request, which therefore holds all its keys; the
 // workgroup normalises and writes the attention's output itself, and no combine pass follows.
-template <typename T, bool WHOLE>
+template <typename T, bool WHOLE, bool SHAPED>
 __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
     const T* __restrict__ q, int q_stride, const void* kpool, const void* vpool,
     const int32_t* __restrict__ block_tables, int max_blocks, const int32_t* __restrict__ q_start,
@@ -1147,8 +1146,7 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
   const int col = lane % 16;
   const bool col_valid = h0 + col < g;
   const int head = kvh * g + h0 + (col_valid ? col : 0);
-  const ScoreShape shape = score_shape(cap, slopes, head);
-  const bool shaped = __builtin_amdgcn_ballot_w64(shape.any()) != 0;   // the same in every lane
+  const ScoreShape shape = SHAPED ? score_shape(cap, slopes, head) : ScoreShape();
   const size_t token = q_start[seq];
 
   Frag<T> qf[kSteps];
@@ -1229,8 +1227,8 @@ __global__ __launch_bounds__(kDecodeWaves* kWave) void attn_decode_kernel(
       for (int u = 0; u < kDecodeDepth; ++u) load_k_of(u, kb_next + 16 * u);
     }
     Frag<T> pf[kDecodeDepth];
-    if (shaped) shape_scores<kDecodeDepth, sizeof(T) == 4>(s, scale_log2, kb0, pos, lane, shape);
-    const float sm_scale = shaped ? 1.0f : scale_log2;
+    if constexpr (SHAPED) shape_scores<kDecodeDepth, sizeof(T) == 4>(s, scale_log2, kb0, pos, lane, shape);
+    const float sm_scale = SHAPED ? 1.0f : scale_log2;
     if (aligned && kb0 >= lo && kb0 + GK <= k_end)
       softmax_group<T, false, kDecodeDepth>(s, pf, sm_scale, kb0, pos, window, keep, k_end, st, o, lane);
     else
@@ -1469,10 +1467,16 @@ int lyp_attn_prefill(const void* q, int q_stride, void* out, int out_stride, con
   do {                                                                                                      \
     constexpr int kQW = (4 / GH) * QB * 16;                                                                 \
     dim3 grid(n_tiles*(64 / kQW), nkv * head_groups);                                                      \
-    attn_prefill_kernel<T, GH, QB><<<grid, 256, 0, stream>>>(                                               \
-        static_cast<const T*>(q), q_stride, static_cast<T*>(out), out_stride, kpool, vpool, block_tables,   \
-        max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window, scale_log2, keep,    \
-        sink, cap, slopes);                                                                                 \
+    if (cap > 0.f || slopes != nullptr)                                                                     \
+      attn_prefill_kernel<T, GH, QB, true><<<grid, 256, 0, stream>>>(                                       \
+          static_cast<const T*>(q), q_stride, static_cast<T*>(out), out_stride, kpool, vpool, block_tables, \
+          max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window, scale_log2, keep,  \
+          sink, cap, slopes);                                                                               \
+    else                                                                                                    \
+      attn_prefill_kernel<T, GH, QB, false><<<grid, 256, 0, stream>>>(                                      \
+          static_cast<const T*>(q), q_stride, static_cast<T*>(out), out_stride, kpool, vpool, block_tables, \
+          max_blocks, q_start, ctx_len, tile_seq, tile_q0, n_tiles, nh, nkv, bs, window, scale_log2, keep,  \
+          sink, cap, slopes);                                                                               \
   } while (0)
 #define LYP_PREFILL_T(T)                    \
   do {                                      \
@@ -1566,11 +1570,16 @@ int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, cons
   dim3 grid(max_parts, nkv * col_groups, n_seqs);
   dim3 cgrid(nh, n_seqs);
   const float scale_log2 = scale * kLog2e;
-#define LYP_DECODE(T, WHOLE)                                                                             \
-  attn_decode_kernel<T, WHOLE><<<grid, kDecodeWaves * kWave, lds, stream>>>(                            \
+#define LYP_DECODE_S(T, WHOLE, SH)                                                                       \
+  attn_decode_kernel<T, WHOLE, SH><<<grid, kDecodeWaves * kWave, lds, stream>>>(                        \
       static_cast<const T*>(q), q_stride, kpool, vpool, block_tables, max_blocks, q_start, ctx_len,      \
       dec_seqs, part_o, part_ml, max_parts, keys_per_wave, nh, nkv, bs, window, scale_log2,              \
       static_cast<T*>(out), out_stride, keep, sink, cap, slopes)
+#define LYP_DECODE(T, WHOLE)                                                \
+  do {                                                                      \
+    if (cap > 0.f || slopes != nullptr) LYP_DECODE_S(T, WHOLE, true);       \
+    else LYP_DECODE_S(T, WHOLE, false);                                     \
+  } while (0)
 #define LYP_DECODE_T(T)                                                                                  \
   do {                                                                                                   \
     if (whole) {                                                                                         \
@@ -1590,6 +1599,7 @@ int lyp_attn_decode(const void* q, int q_stride, void* out, int out_stride, cons
     LYP_REQUIRE(false, "attn_decode: unknown dtype %d", dtype);
   }
 #undef LYP_DECODE_T
+#undef LYP_DECODE_S
 #undef LYP_DECODE
   LYP_LAUNCH_CHECK("attn_decode");
   return 0;
