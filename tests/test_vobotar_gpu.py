@@ -16,7 +16,7 @@ import torch
 from conftest import ROOT
 from trace_util import Trace, compare, compare_with_alone, random_tokens, random_trace, replay
 from vobotar_util import (BLOCK_SIZE, CONFIGS, RANKS, attention, config, dense, edit, pair, pair2, plain_greedy, plain_logits,
-                          plain_sensitivity, write_model)
+                          plain_sensitivity, random_config, write_model)
 
 pytestmark = pytest.mark.gpu
 DTYPES = ["float32", "bfloat16"]
@@ -370,6 +370,21 @@ def test_other_orders_and_sizes(tmp_path, dtype, layers):
         t.step([("x", 1), ("y", 1)])
     t.step([("x", 45)], end=["x", "y"])
     check_folder(t, replay(folder, dtype, t, block_size=16 if "heads of" in layers else 8), folder, dtype, layers)
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations_under_random_schedules(tmp_path, seed):
+    """Configurations and schedules drawn at random, in 32-bit, where the engine must agree with the
+    plain model to 1e-4 of the largest logit and what a row's own sensitivity explains (a 32-bit
+    rounding step is 2^-15 of the 16-bit one that ``plain_sensitivity`` measures)."""
+    rng = random.Random(9000 + seed)
+    cfg = random_config(rng)
+    folder = write_model(str(tmp_path / "m"), cfg, seed=seed, dtype="float32", rank=rng.choice([3, 8, 16]))
+    reqs, t = random_trace(rng, cfg["vocab"], rng.choice([60, 150, 300]))
+    got = replay(folder, "float32", t, block_size=rng.choice([4, 8, 16]), num_state_slots=4)
+    slack = {rid: 16.0 * 2.0 ** -15 * s.numpy() for rid, s in plain_sensitivity(folder, t.requests).items()}
+    compare(t, got, plain_logits(folder, t.requests), "float32", f"random configuration {seed}", tol=dict(rtol=1e-4, atol=1e-4),
+            slack=slack)
 
 
 # ------------------------------------------------------------------- generation

@@ -58,6 +58,45 @@ def config(vocab, width, layers, *, eps=1e-6, scale=1.0, side=0):
     return d
 
 
+def random_config(rng) -> dict:
+    """A configuration drawn at random: width, vocabulary, one to six layers of any kind in any
+    order, heads and key/value heads, key and value sizes that are equal or not (the matrix-core
+    kernels or the row-by-row one), windows from one token up, rotations of two values up to the
+    whole head, caps, blended values, taps, groups, with and without feed-forward and side input."""
+    def divisors(n):
+        return [d for d in range(1, n + 1) if n % d == 0]
+
+    width = rng.choice([48, 64, 96, 128, 160, 192, 256])
+    sizes = [8, 16, 24, 32, 48, 64, 80, 96, 128]
+    g_att, vd_att = rng.choice([1, 2, 4]), rng.choice([8, 16, 32, 48, 64])     # blending layers share the values' shape
+    layers = []
+    for _ in range(rng.randint(1, 6)):
+        kind = rng.choice(["attention", "parallel", "parallel_2"])
+        mlp = None if rng.random() < 0.2 else dense(rng.choice([32, 64, 100, 192, 320]))
+        scale = lambda d: round(d ** -0.5 * rng.uniform(0.7, 2.0), 4)
+        if kind == "attention":
+            d = vd_att if rng.random() < 0.4 else rng.choice(sizes)
+            rot = None if rng.random() < 0.2 else (rng.choice([100.0, 1e4, 1e6]), rng.choice(range(2, d + 1, 2)))
+            layers.append(attention(g_att * rng.choice([1, 2, 3, 4]), g_att, d, vd_att, scale(d), rot=rot,
+                                    softcap=rng.choice([None, 5.0, 20.0, 50.0]), v_mix=rng.random() < 0.7, mlp=mlp))
+        elif kind == "parallel":
+            g, d = rng.choice([1, 2, 4, 8]), rng.choice(sizes[:8])
+            layers.append(pair((g * rng.choice([1, 2, 3]), g, d, scale(d), rng.choice([None, 1, 7, 16, 33, 72, 150])),
+                               (rng.choice([1, 2, 3, 4]), rng.choice([8, 16, 24, 48, 64, 100])),
+                               round(rng.uniform(0.3, 1.5), 2), round(rng.uniform(0.3, 1.5), 2), mlp=mlp))
+        else:
+            g, d = rng.choice([1, 2, 4]), rng.choice(sizes)
+            dv = d if rng.random() < 0.6 else rng.choice(sizes)
+            rot = None if rng.random() < 0.2 else (rng.choice([100.0, 2.5e5]), rng.choice(range(2, d + 1, 2)))
+            heads = rng.choice([1, 2, 4, 6])
+            layers.append(pair2((g * rng.choice([1, 2, 3]), g, d, dv, scale(d), rng.choice([None, 2, 9, 31, 64, 136]), rot),
+                                (heads, rng.choice([8, 16, 32]), rng.choice([8, 16, 48, 64, 100]), rng.choice(divisors(heads)),
+                                 rng.choice([1, 2, 3, 4, 5]), rng.choice(divisors(heads))),
+                                round(rng.uniform(0.3, 1.5), 2), round(rng.uniform(0.3, 1.5), 2), mlp=mlp))
+    return config(rng.randint(100, 600), width, layers, eps=rng.choice([1e-6, 1e-5]), scale=rng.choice([0.5, 1.0, 2.0]),
+                  side=rng.choice([0, 4, 12, 16, 32]))
+
+
 # Three configurations that differ in every size and option; none of their sizes coincide where a
 # model's might by chance (key and value sizes, heads and key heads, heads x value size and width).
 #   A: odd sizes (the row-by-row attention, the scalar paths): keys of 10 with values of 12, one
